@@ -106,18 +106,18 @@ class TorchOps:
 
     def attend(self, qkv, batch, table, cache, write_cache, *, num_heads, num_kv_heads,
                kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window,
-               defer_merge=False):
+               defer_merge=False, sink=None):
         q = self.qk_norm_rope_store(
             qkv, batch, table, cache if write_cache else None, num_heads=num_heads,
             num_kv_heads=kv_in_row, head_dim=head_dim, q_weight=q_weight, k_weight=k_weight,
             eps=eps, cos_sin=cos_sin)
         return self.paged_attention(q, batch, table, cache, num_heads=num_heads,
                                     num_kv_heads=num_kv_heads, head_dim=head_dim,
-                                    scale=scale, window=window)
+                                    scale=scale, window=window, sink=sink)
 
     # ---------------------------------------------------------------- attention
     def paged_attention(self, q, batch, table, cache, *, num_heads, num_kv_heads, head_dim,
-                        scale, window, only=None):
+                        scale, window, only=None, sink=None):
         """`only`: compute just these flat tokens (a test's choice; the other rows of the
         result are left unset)."""
         T = q.shape[0]
@@ -136,7 +136,11 @@ class TorchOps:
             v = cache.v_pages[pages, :, :, keys % P].float()
             for j in range(num_heads):
                 s = (k[:, j // group] @ q[t, j].float()) * scale
-                out[t, j] = torch.softmax(s, dim=0) @ v[:, j // group]
+                if sink is None:
+                    out[t, j] = torch.softmax(s, dim=0) @ v[:, j // group]
+                else:       # one more score in the denominator, with nothing to add
+                    w = torch.softmax(torch.cat([s, sink[j].float().view(1)]), dim=0)
+                    out[t, j] = w[:-1] @ v[:, j // group]
         return out.to(q.dtype)
 
     # ---------------------------------------------------------------- stream norms, shift
@@ -277,9 +281,11 @@ class TorchOps:
         return (yf.view(T, inner) * act).to(out_dtype)
 
     # ---------------------------------------------------------------- routed experts
-    def route_experts(self, logits, *, top, group_count, group_keep):
+    def route_experts(self, logits, *, top, group_count=1, group_keep=1, scores="softmax",
+                      normalize=True):
         T, E = logits.shape
-        scores = torch.softmax(logits.float(), dim=-1)
+        scores = torch.softmax(logits.float(), dim=-1) if scores == "softmax" \
+            else torch.sigmoid(logits.float())
         per = E // group_count
         best = scores.view(T, group_count, per).max(-1).values
         kept = torch.zeros(T, group_count, dtype=torch.bool, device=logits.device)
@@ -288,21 +294,61 @@ class TorchOps:
         chosen = torch.where(allowed, scores, torch.full_like(scores, -1.0)).topk(top, -1).indices
         picked = torch.gather(scores, 1, chosen)
         out = torch.zeros_like(scores)
-        out.scatter_(1, chosen, picked / (picked.sum(-1, keepdim=True) + 1e-20))
+        out.scatter_(1, chosen, picked / (picked.sum(-1, keepdim=True) + 1e-20)
+                     if normalize else picked)
         return out
 
-    def expert_activation(self, gate_up, weights, inner, limit, out_dtype):
+    def expert_activation(self, gate_up, weights, inner, limit, out_dtype, weighted_input=False):
         T, E = weights.shape
         gu = gate_up.float().view(T, E, 2, inner)
+        if weighted_input:
+            w = weights.float()[:, :, None]
+            g, u = gu[:, :, 0] * w, gu[:, :, 1] * w
+            return (g * torch.sigmoid(g) * u).view(T, E * inner).to(out_dtype)
         g = torch.clamp(gu[:, :, 0], max=limit)
         u = torch.clamp(gu[:, :, 1], -limit, limit)
         y = g * torch.sigmoid(1.702 * g) * (u + 1.0) * weights.float()[:, :, None]
         return y.view(T, E * inner).to(out_dtype)
 
+    # ---------------------------------------------------------------- gated diagonal recurrence
+    def rglru_gates(self, u, w_a, w_i, b_a, b_i, rate):
+        T, width = u.shape
+        blocks, bw = w_a.shape[0], w_a.shape[1]
+        ub = u.float().view(T, blocks, bw)
+        r = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, w_a.float()).reshape(T, width) + b_a)
+        i = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, w_i.float()).reshape(T, width) + b_i)
+        log_a = rate * r
+        return torch.exp(log_a), torch.sqrt(-torch.expm1(2.0 * log_a)) * i * u.float()
+
+    def rglru_scan(self, a, x, proj, y_col, y_bias, batch, state, out_dtype):
+        T, width = a.shape
+        y = proj[:, y_col:y_col + width].float()
+        if y_bias is not None:
+            y = y + y_bias
+        gate = 0.5 * y * (1.0 + torch.tanh(0.7978845608028654 * (y + 0.044715 * y ** 3)))
+        out = torch.empty(T, width, dtype=torch.float32, device=a.device)
+        for b, lo, hi, slot, start in self._entries(batch):
+            S = state[slot].clone() if start > 0 else torch.zeros_like(state[slot])
+            for t in range(lo, hi):
+                S = a[t] * S + x[t]
+                out[t] = S
+            state[slot] = S
+        return (out * gate).to(out_dtype)
+
+    def relu_squared(self, x, out_dtype):
+        return torch.relu(x.float()).pow(2).to(out_dtype)
+
+    def sigmoid_gate(self, x, gate_rows, gate_col, out_dtype):
+        n = x.shape[1]
+        return (x.float() * torch.sigmoid(gate_rows[:, gate_col:gate_col + n].float())).to(out_dtype)
+
     # ---------------------------------------------------------------- state-space mixer
-    def conv_silu(self, proj, col, channels, weight, bias, batch, state):
+    def conv_silu(self, proj, col, channels, weight, bias, batch, state, in_bias=None,
+                  plain=False):
         taps = weight.shape[1]
         u = proj[:, col:col + channels].float()
+        if in_bias is not None:
+            u = u + in_bias.float()
         out = torch.empty_like(u)
         for b, lo, hi, slot, start in self._entries(batch):
             hist = state[slot] if start > 0 else torch.zeros_like(state[slot])
@@ -312,7 +358,7 @@ class TorchOps:
                 else torch.zeros(n, channels, dtype=torch.float32, device=u.device)
             for k in range(taps):
                 acc = acc + full[k:k + n] * weight[:, k].float()
-            out[lo:hi] = acc * torch.sigmoid(acc)
+            out[lo:hi] = acc if plain else acc * torch.sigmoid(acc)
             if taps > 1:
                 state[slot] = full[full.shape[0] - (taps - 1):]
         return out

@@ -111,7 +111,8 @@ __device__ __forceinline__ float load_past_caches(const float* p) {
 // uses the first.
 template <int HD, int THREADS>
 __device__ __forceinline__ void merge_splits_here(const float* partial_o, const float* partial_ml,
-                                                  int64_t first_slot, int used, int rows, bf16_t* out) {
+                                                  int64_t first_slot, int used, int rows, bf16_t* out,
+                                                  const float* sink = nullptr, int first_head = 0) {
   constexpr int kGroup = 8, E = 2;
   const int count = rows * HD;
   for (int e0 = threadIdx.x; e0 < count; e0 += E * THREADS) {
@@ -158,7 +159,8 @@ __device__ __forceinline__ void merge_splits_here(const float* partial_o, const 
 #pragma unroll
     for (int k = 0; k < E; ++k) {
       if (e0 + k * THREADS >= count) break;
-      const float inv = L[k] > 0.f ? 1.f / L[k] : 0.f;
+      const float sum = sum_with_sink(L[k], M[k], sink, first_head + row[k]);
+      const float inv = sum > 0.f ? 1.f / sum : 0.f;
       out[(int64_t)row[k] * HD + d[k]] = (bf16_t)(acc[k] * inv);
     }
   }
@@ -379,7 +381,9 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
     }
     m = M;
     // lane (r, g) holds O^T[d = db*16 + g*4 + i][row r]
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    // the sink joins the sum where the row is finished: here only without key splits
+    const float whole = ma.num_splits == 1 ? sum_with_sink(l, m, a.sink, head) : l;
+    const float inv = whole > 0.f ? 1.f / whole : 0.f;
 #pragma unroll
     for (int k = 0; k < kShare; ++k) {
       const int db = wave * kShare + k;
@@ -431,7 +435,7 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
   const int rows = min(ma.rows_per_token, group - hb * 16);
   bf16_t* out = (bf16_t*)a.out + ((int64_t)token * a.nq + kvh * group + hb * 16) * HD;
   merge_splits_here<HD, NW * kWave>(ma.partial_o, ma.partial_ml, (int64_t)item * ma.num_splits * 16,
-                                    used, rows, out);
+                                    used, rows, out, a.sink, kvh * group + hb * 16);
 }
 
 int ts_check_attention_mfma_args(const AttentionMfmaArgs& args, const char* who);

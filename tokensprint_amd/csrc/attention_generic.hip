@@ -149,6 +149,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
     weight[w] = m_s[w] == -INFINITY ? 0.f : expf(m_s[w] - m_all);     // a wavefront without keys
     l += l_s[w] * weight[w];
   }
+  if (a.sink) l += expf(fminf(a.sink[item % a.nq] - m_all, 69.f));    // the head's sink
   T* o = (T*)a.out + item * hd;
   const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll

@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attention_mfma_kernel(
   // lane (r, g) holds O^T[d = db*16 + g*4 + i][row r]
   if (args.num_splits == 1) {
     if (!row_ok) return;
-    store_tile<HD>(t, l, (bf16_t*)a.out + ((int64_t)token * a.nq + head) * HD, g);
+    store_tile<HD>(t, sum_with_sink(l, m, a.sink, head), (bf16_t*)a.out + ((int64_t)token * a.nq + head) * HD, g);
   } else {
     const int64_t slot = ((int64_t)item * args.num_splits + split) * 16 + r;
     if (row_ok) {
@@ -214,6 +214,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttentionMfmaArgs 
     }
     M = Mg;
   }
+  L = sum_with_sink(L, M, a.sink, kvh * group + hh);
   const float inv = L > 0.f ? 1.f / L : 0.f;
   bf16_t* out = (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + kvh * group + hh) * HD;
 #pragma unroll

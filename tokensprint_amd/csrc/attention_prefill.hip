@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionMfmaArg
 
 #pragma unroll
   for (int j = 0; j < TPW; ++j) {
-    const float sum = row_sum<HD>(ts[j]);        // by all lanes: it crosses lanes
+    const float sum = sum_with_sink(row_sum<HD>(ts[j]), ts[j].m, a.sink, head);        // by all lanes: it crosses lanes
     if (ts[j].pos < 0) continue;
     store_tile<HD>(ts[j], sum,
                    (bf16_t*)a.out + ((int64_t)(tok0 + j * tq + ti) * a.nq + head) * HD, g);
@@ -302,7 +302,7 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
       buf ^= 1;
     }
   }
-  const float sum = row_sum<HD>(t);                // by all lanes: it crosses lanes
+  const float sum = sum_with_sink(row_sum<HD>(t), t.m, a.sink, head);                // by all lanes: it crosses lanes
   if (row_ok)
     store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
 }
@@ -538,12 +538,12 @@ __global__ __launch_bounds__(256 * H, H == 1 ? 3 : 2) void attention_prefill_asy
             const float o1 = lds_o[((wave * DB + db) * 4 + i) * kWave + lane];
             t.o[db][i] = t.o[db][i] * w0 + (w1 == 0.f ? 0.f : o1 * w1);
           }
-        const float sum = row_sum<HD>(t);          // by all lanes: it crosses lanes
+        const float sum = sum_with_sink(row_sum<HD>(t), t.m, a.sink, head);          // by all lanes: it crosses lanes
         if (row_ok)
           store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
       }
     } else {
-      const float sum = row_sum<HD>(t);            // by all lanes: it crosses lanes
+      const float sum = sum_with_sink(row_sum<HD>(t), t.m, a.sink, head);            // by all lanes: it crosses lanes
       if (row_ok)
         store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
     }
@@ -911,12 +911,12 @@ __device__ __forceinline__ void attention_prefill_wide(const AttentionMfmaArgs& 
             const float o1 = lds_o[((wave * DB + db) * 4 + i) * kWave + lane];
             t.o[db][i] = t.o[db][i] * w0 + (w1 == 0.f ? 0.f : o1 * w1);
           }
-        const float sum = row_sum<HD>(t);
+        const float sum = sum_with_sink(row_sum<HD>(t), t.m, a.sink, head);
         if (row_ok)
           store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
       }
     } else {
-      const float sum = row_sum<HD>(t);
+      const float sum = sum_with_sink(row_sum<HD>(t), t.m, a.sink, head);
       if (row_ok)
         store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
     }

@@ -7,9 +7,11 @@
 // the `group_keep` best groups' experts can be chosen; of those the `top` with the largest
 // scores (equal scores: the lower index).  weights[t][e] = score / (sum of the chosen scores
 // + 1e-20) for the chosen experts and 0 for the others.
+// `sigmoid_scores`: scores = sigmoid(logits), each expert by itself, instead of the softmax;
+// `normalize` 0: the weights are the chosen experts' scores as they are.
 __global__ __launch_bounds__(256) void route_experts_kernel(
     const float* __restrict__ logits, float* __restrict__ weights, int rows, int E, int top,
-    int group_count, int group_keep) {
+    int group_count, int group_keep, int sigmoid_scores, int normalize) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;
@@ -18,19 +20,23 @@ __global__ __launch_bounds__(256) void route_experts_kernel(
   float* open = score + E;                       // the score while the expert can be chosen, else -1
   float* best = open + E;                        // [group_count]
   const float* z = logits + (live ? t : 0) * E;
-  float m = -INFINITY;
-  for (int e = lane; e < E; e += kWave) m = fmaxf(m, z[e]);
-  m = wave_max(m);
-  float sum = 0.f;
-  for (int e = lane; e < E; e += kWave) {
-    const float p = expf(z[e] - m);
-    score[e] = p;
-    sum += p;
-  }
-  sum = wave_sum(sum);
-  const float inv = 1.0f / sum;
   const int per = E / group_count;
-  for (int e = lane; e < E; e += kWave) score[e] *= inv;
+  if (sigmoid_scores) {
+    for (int e = lane; e < E; e += kWave) score[e] = 1.0f / (1.0f + expf(-z[e]));
+  } else {
+    float m = -INFINITY;
+    for (int e = lane; e < E; e += kWave) m = fmaxf(m, z[e]);
+    m = wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += kWave) {
+      const float p = expf(z[e] - m);
+      score[e] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+    for (int e = lane; e < E; e += kWave) score[e] *= inv;
+  }
   __syncthreads();
   for (int g = lane; g < group_count; g += kWave) {
     float b = -1.f;
@@ -65,13 +71,14 @@ __global__ __launch_bounds__(256) void route_experts_kernel(
     }
     __syncthreads();
   }
-  const float norm = 1.0f / (chosen_sum + 1e-20f);
+  const float norm = normalize ? 1.0f / (chosen_sum + 1e-20f) : 1.0f;
   if (live)
     for (int e = lane; e < E; e += kWave) w[e] = open[e] == -2.f ? score[e] * norm : 0.f;
 }
 
 extern "C" int ts_route_experts(const float* logits, float* weights, int rows, int experts,
-                                int top, int group_count, int group_keep, hipStream_t stream) {
+                                int top, int group_count, int group_keep, int sigmoid_scores,
+                                int normalize, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (experts <= 0 || group_count <= 0 || experts % group_count || group_keep <= 0 ||
       group_keep > group_count || top <= 0 || top > group_keep * (experts / group_count))
@@ -80,7 +87,7 @@ extern "C" int ts_route_experts(const float* logits, float* weights, int rows, i
   const size_t lds = (size_t)4 * (2 * experts + group_count) * sizeof(float);
   if (lds > 64 * 1024) TS_FAIL("route_experts: %d experts are more than the kernel holds", experts);
   hipLaunchKernelGGL(route_experts_kernel, dim3((rows + 3) / 4), dim3(256), lds, stream, logits,
-                     weights, rows, experts, top, group_count, group_keep);
+                     weights, rows, experts, top, group_count, group_keep, sigmoid_scores, normalize);
   TS_CHECK_LAUNCH("route_experts");
   return 0;
 }
@@ -89,10 +96,12 @@ extern "C" int ts_route_experts(const float* logits, float* weights, int rows, i
 // gate_up [rows, E, gate | up] (inner columns each) -> out [rows, E, inner]:
 // g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(1.702 g) (u + 1) times
 // the token's weight for the expert; zeros (and no reads) where the weight is zero.
+// `weighted_input`: the expert is a plain gated unit whose input was the token times its
+// weight w, and both products are linear in it: out = silu(w gate) (w up).
 template <typename T>
 __global__ __launch_bounds__(256) void expert_activation_kernel(
     const T* __restrict__ gate_up, const float* __restrict__ weights, T* __restrict__ out,
-    int64_t total, int E, int inner, float limit) {
+    int64_t total, int E, int inner, float limit, int weighted_input) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const int64_t te = idx / inner;                 // token * E + expert
@@ -101,6 +110,11 @@ __global__ __launch_bounds__(256) void expert_activation_kernel(
   float y = 0.f;
   if (w != 0.f) {
     const T* src = gate_up + te * 2 * inner;
+    if (weighted_input) {
+      const float g = w * to_f32(src[i]), u = w * to_f32(src[inner + i]);
+      out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+      return;
+    }
     const float g = fminf(to_f32(src[i]), limit);
     const float u = fminf(fmaxf(to_f32(src[inner + i]), -limit), limit);
     y = g / (1.0f + expf(-1.702f * g)) * (u + 1.0f) * w;
@@ -110,7 +124,7 @@ __global__ __launch_bounds__(256) void expert_activation_kernel(
 
 extern "C" int ts_expert_activation(const void* gate_up, const float* weights, void* out, int type,
                                     int rows, int experts, int inner, float limit,
-                                    hipStream_t stream) {
+                                    int weighted_input, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (experts <= 0 || inner <= 0) TS_FAIL("expert_activation: bad sizes");
   const int64_t total = (int64_t)rows * experts * inner;
@@ -118,7 +132,7 @@ extern "C" int ts_expert_activation(const void* gate_up, const float* weights, v
                    hipLaunchKernelGGL(expert_activation_kernel<T>,
                                       dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
                                       (const T*)gate_up, weights, (T*)out, total, experts, inner,
-                                      limit));
+                                      limit, weighted_input));
   TS_CHECK_LAUNCH("expert_activation");
   return 0;
 }

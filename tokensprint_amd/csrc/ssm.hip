@@ -24,11 +24,16 @@ __device__ __forceinline__ float softplus_f(float v) { return v > 20.f ? v : log
 // the sequence are zero, inputs in front of the portion come from state[slot][taps-1][C],
 // whose row j holds the input at position start - (taps-1) + j.
 
+// `in_bias` (may be null): added to every input of the sequence before the convolution (the
+// zeros in front of the sequence stay zeros; the state holds inputs with it added).
+// `plain` 1: no activation behind the convolution.
+
 // One thread per (token, channel); writes no state.
 __global__ __launch_bounds__(256) void conv_silu_kernel(
     const float* __restrict__ proj, int ld, int col, int channels, int taps,
     const float* __restrict__ w, const float* __restrict__ bias, const float* __restrict__ state,
-    float* __restrict__ out, BatchView b, int num_tokens) {
+    float* __restrict__ out, BatchView b, int num_tokens, const float* __restrict__ in_bias,
+    int plain) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (int64_t)num_tokens * channels) return;
   const int t = (int)(idx / channels), c = (int)(idx % channels);
@@ -36,15 +41,16 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(
   const int first = b.q_start[e], pos = b.positions[t];
   const float* st = state + (int64_t)b.slot_ids[e] * (taps - 1) * channels;
   float acc = bias ? bias[c] : 0.f;
+  const float ib = in_bias ? in_bias[c] : 0.f;
   for (int k = 0; k < taps; ++k) {
     const int back = taps - 1 - k;
     if (pos - back < 0) continue;
     float v;
-    if (t - back >= first) v = proj[(int64_t)(t - back) * ld + col + c];
+    if (t - back >= first) v = proj[(int64_t)(t - back) * ld + col + c] + ib;
     else v = st[(int64_t)(taps - 1 - (first - (t - back))) * channels + c];
     acc = fmaf(w[c * taps + k], v, acc);
   }
-  out[(int64_t)t * channels + c] = silu_f(acc);
+  out[(int64_t)t * channels + c] = plain ? acc : silu_f(acc);
 }
 
 // One thread per (entry, channel): the state after the portion.  Row j takes the input at
@@ -52,7 +58,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(
 // any row at or above it is written: j ascends), or zero in front of the sequence.
 __global__ __launch_bounds__(256) void conv_state_kernel(
     const float* __restrict__ proj, int ld, int col, int channels, int taps,
-    float* __restrict__ state, BatchView b, int num_entries) {
+    float* __restrict__ state, BatchView b, int num_entries, const float* __restrict__ in_bias) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (int64_t)num_entries * channels) return;
   const int e = (int)(idx / channels), c = (int)(idx % channels);
@@ -62,7 +68,7 @@ __global__ __launch_bounds__(256) void conv_state_kernel(
   for (int j = 0; j < taps - 1; ++j) {
     const int p = start + n - (taps - 1) + j;
     float v = 0.f;
-    if (p >= start) v = proj[(int64_t)(first + p - start) * ld + col + c];
+    if (p >= start) v = proj[(int64_t)(first + p - start) * ld + col + c] + (in_bias ? in_bias[c] : 0.f);
     else if (p >= 0) v = st[(int64_t)(j + n) * channels + c];
     st[(int64_t)j * channels + c] = v;
   }
@@ -74,11 +80,13 @@ constexpr int kMaxTapsInRegisters = 8;
 __global__ __launch_bounds__(256) void conv_silu_walk_kernel(
     const float* __restrict__ proj, int ld, int col, int channels, int taps,
     const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ state,
-    float* __restrict__ out, BatchView b, int num_entries) {
+    float* __restrict__ out, BatchView b, int num_entries, const float* __restrict__ in_bias,
+    int plain) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (int64_t)num_entries * channels) return;
   const int e = (int)(idx / channels), c = (int)(idx % channels);
   const int first = b.q_start[e], end = b.q_start[e + 1];
+  const float ib = in_bias ? in_bias[c] : 0.f;
   const int start = b.positions[first];
   float* st = state + (int64_t)b.slot_ids[e] * (taps - 1) * channels;
   float hist[kMaxTapsInRegisters], wk[kMaxTapsInRegisters];
@@ -91,14 +99,14 @@ __global__ __launch_bounds__(256) void conv_silu_walk_kernel(
   }
   const float bc = bias ? bias[c] : 0.f;
   for (int t = first; t < end; ++t) {
-    const float v = proj[(int64_t)t * ld + col + c];
+    const float v = proj[(int64_t)t * ld + col + c] + ib;
     float acc = bc;
 #pragma unroll
     for (int k = 0; k < kMaxTapsInRegisters; ++k) {
       if (k < taps - 1) acc = fmaf(wk[k], hist[k], acc);
       else if (k == taps - 1) acc = fmaf(wk[k], v, acc);
     }
-    out[(int64_t)t * channels + c] = silu_f(acc);
+    out[(int64_t)t * channels + c] = plain ? acc : silu_f(acc);
 #pragma unroll
     for (int k = 0; k < kMaxTapsInRegisters - 1; ++k) {
       if (k < taps - 2) hist[k] = hist[k + 1];
@@ -114,7 +122,7 @@ extern "C" int ts_conv_silu(const float* proj, int ld, int col, int channels, in
                             const float* w, const float* bias, float* state, float* out,
                             const int* positions, const int* entry_of_token, const int* q_start,
                             const int* slot_ids, int num_tokens, int num_entries, int max_q_len,
-                            hipStream_t stream) {
+                            const float* in_bias, int plain, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (channels <= 0 || taps < 1 || col < 0 || col + channels > ld)
     TS_FAIL("conv_silu: bad sizes channels=%d taps=%d col=%d ld=%d", channels, taps, col, ld);
@@ -123,18 +131,18 @@ extern "C" int ts_conv_silu(const float* proj, int ld, int col, int channels, in
     const int64_t n = (int64_t)num_entries * channels;
     hipLaunchKernelGGL(conv_silu_walk_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                        stream, proj, ld, col, channels, taps, w, bias, state, out, b,
-                       num_entries);
+                       num_entries, in_bias, plain);
     TS_CHECK_LAUNCH("conv_silu (walk)");
     return 0;
   }
   const int64_t n = (int64_t)num_tokens * channels;
   hipLaunchKernelGGL(conv_silu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
-                     proj, ld, col, channels, taps, w, bias, state, out, b, num_tokens);
+                     proj, ld, col, channels, taps, w, bias, state, out, b, num_tokens, in_bias, plain);
   TS_CHECK_LAUNCH("conv_silu");
   if (taps > 1) {
     const int64_t m = (int64_t)num_entries * channels;
     hipLaunchKernelGGL(conv_state_kernel, dim3((unsigned)((m + 255) / 256)), dim3(256), 0, stream,
-                       proj, ld, col, channels, taps, state, b, num_entries);
+                       proj, ld, col, channels, taps, state, b, num_entries, in_bias);
     TS_CHECK_LAUNCH("conv_state");
   }
   return 0;

@@ -9,7 +9,7 @@ library, construction raises.
 from __future__ import annotations
 
 import ctypes
-from ctypes import Structure, byref, c_float, c_int, c_void_p
+from ctypes import Structure, byref, c_float, c_int, c_int64, c_void_p
 
 import numpy as np
 import torch
@@ -48,7 +48,7 @@ class AttentionArgs(Structure):
         ("ctx_len", c_void_p), ("table", c_void_p),
         ("table_width", c_int), ("num_tokens", c_int), ("num_entries", c_int), ("nq", c_int),
         ("nkv", c_int), ("hd", c_int), ("page_size", c_int), ("num_pages", c_int),
-        ("window", c_int), ("scale", c_float),
+        ("window", c_int), ("scale", c_float), ("sink", c_void_p),
     ]
 
 
@@ -669,7 +669,9 @@ class HipOps:
 
     # ------------------------------------------------------------ attention
     def paged_attention(self, q, batch, table, cache, *, num_heads, num_kv_heads, head_dim,
-                        scale, window):
+                        scale, window, sink=None):
+        """`sink`: float32 [num_heads] or None: a score per query head that joins the
+        softmax's denominator once (not scaled, no key, no value)."""
         T = q.shape[0]
         self._check("q", q, self._FLOATS, shape=(T, num_heads, head_dim))
         self._check_cache(cache, table, batch, num_kv_heads, head_dim)
@@ -678,7 +680,7 @@ class HipOps:
         out = torch.empty_like(q)
         a = AttentionArgs()
         self._fill_attention_args(a, q, out, batch, table, cache, num_heads, num_kv_heads,
-                                  head_dim, scale, window)
+                                  head_dim, scale, window, sink)
         if (q.dtype == torch.bfloat16 and cache.k_pages.dtype == torch.bfloat16
                 and head_dim % 16 == 0 and head_dim <= 256 and cache.page_size % 4 == 0):
             if self._decode_fits(batch, num_kv_heads, num_heads // num_kv_heads, head_dim,
@@ -693,7 +695,7 @@ class HipOps:
 
     def attend(self, qkv, batch, table, cache, write_cache, *, num_heads, num_kv_heads,
                kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window,
-               defer_merge=False):
+               defer_merge=False, sink=None):
         """Everything between the q/k/v projection and the output projection: per-head
         norm of q and k, rotation, the write of k and v into `cache` (if `write_cache`;
         the row then brings `kv_in_row` = `num_kv_heads` key and value heads) and attention
@@ -714,7 +716,7 @@ class HipOps:
                 k_weight=k_weight, eps=eps, cos_sin=cos_sin)
             return self.paged_attention(q, batch, table, cache, num_heads=num_heads,
                                         num_kv_heads=num_kv_heads, head_dim=head_dim,
-                                        scale=scale, window=window)
+                                        scale=scale, window=window, sink=sink)
         # the same argument checks as the preparation kernel's
         qa = self._qk_args(qkv, batch, num_heads=num_heads, kv_in_row=kv_in_row,
                            head_dim=head_dim, q_weight=q_weight, k_weight=k_weight, eps=eps,
@@ -725,7 +727,9 @@ class HipOps:
         out = torch.empty(T, num_heads, head_dim, dtype=qkv.dtype, device=self.device)
         a = AttentionArgs()
         self._fill_attention_args(a, None, out, batch, table, cache, num_heads, num_kv_heads,
-                                  head_dim, scale, window)
+                                  head_dim, scale, window, sink)
+        if sink is not None:
+            defer_merge = False        # the product that merges for itself knows no sink
         d = AttentionDecodeArgs()
         d.qkv, d.q_weight, d.k_weight = qa.qkv, qa.q_weight, qa.k_weight
         d.cos, d.sin, d.eps, d.kv_in_row = qa.cos, qa.sin, eps, kv_in_row
@@ -886,8 +890,10 @@ class HipOps:
         return dev
 
     def _fill_attention_args(self, a, q, out, batch, table, cache, num_heads, num_kv_heads,
-                             head_dim, scale, window):
+                             head_dim, scale, window, sink=None):
         T = out.shape[0]
+        if sink is not None:
+            a.sink = self._check("sink", sink, torch.float32, shape=(num_heads,)).data_ptr()
         a.q, a.out = (q.data_ptr() if q is not None else None), out.data_ptr()
         a.k_pages, a.v_pages = cache.k_pages.data_ptr(), cache.v_pages.data_ptr()
         a.positions, a.entry_of_token = batch.positions.data_ptr(), batch.entry_of_token.data_ptr()
@@ -1017,11 +1023,14 @@ class HipOps:
         return out
 
     # ------------------------------------------------------------ state-space mixer
-    def conv_silu(self, proj, col, channels, weight, bias, batch, state):
+    def conv_silu(self, proj, col, channels, weight, bias, batch, state, in_bias=None,
+                  plain=False):
         """Causal convolution per channel over columns [col, col + channels) of `proj`
         (float32 [T, ld]), bias, SiLU -> float32 [T, channels].  weight [channels, taps]
         (the last tap is the current token's); `state` [slots, taps - 1, channels] carries
-        a request's last inputs."""
+        a request's last inputs.  `in_bias` [channels]: added to every input of the sequence
+        before the convolution (the zeros in front of a sequence stay zeros); `plain`: no
+        activation behind it."""
         self._check("proj", proj, torch.float32, ndim=2)
         T, ld = proj.shape
         self._check("conv weight", weight, torch.float32, ndim=2)
@@ -1031,12 +1040,15 @@ class HipOps:
                              f"weight {tuple(weight.shape)}")
         if bias is not None:
             self._check("conv bias", bias, torch.float32, shape=(channels,))
+        if in_bias is not None:
+            self._check("conv input bias", in_bias, torch.float32, shape=(channels,))
         self._check_state("conv state", state, (taps - 1, channels))
         pos, eot, qs, slots = self._batch_ptrs(batch, T)
         out = torch.empty(T, channels, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_conv_silu, _ptr(proj), ld, col, channels, taps, _ptr(weight),
                    _ptr(bias), _ptr(state), _ptr(out), pos, eot, qs, slots, T,
-                   batch.num_entries, int(batch.max_q_len), self._stream())
+                   batch.num_entries, int(batch.max_q_len), _ptr(in_bias), int(bool(plain)),
+                   self._stream())
         return out
 
     def ssm_scan(self, xbc, proj, dt_col, dt_bias, a_log, d_skip, batch, state, *, heads, vdim,
@@ -1187,22 +1199,29 @@ class HipOps:
         return out
 
     # ------------------------------------------------------------ routed experts
-    def route_experts(self, logits, *, top, group_count, group_keep):
+    def route_experts(self, logits, *, top, group_count=1, group_keep=1, scores="softmax",
+                      normalize=True):
         """Router logits (float32 [T, experts]) -> float32 [T, experts]: a token's weight for
         each of its `top` experts (softmax score over the chosen scores' sum), zero elsewhere.
         Only experts of the `group_keep` best of `group_count` groups of neighbours can be
-        chosen (a group's score: its best expert's)."""
+        chosen (a group's score: its best expert's).  `scores` "sigmoid": an expert's score is
+        the sigmoid of its logit; `normalize` False: the weights are the chosen scores as
+        they are."""
+        if scores not in ("softmax", "sigmoid"):
+            raise ValueError(f"route_experts: scores={scores!r}")
         self._check("router logits", logits, torch.float32, ndim=2)
         T, E = logits.shape
         weights = torch.empty(T, E, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_route_experts, _ptr(logits), _ptr(weights), T, E, int(top),
-                   int(group_count), int(group_keep), self._stream())
+                   int(group_count), int(group_keep), int(scores == "sigmoid"),
+                   int(bool(normalize)), self._stream())
         return weights
 
-    def expert_activation(self, gate_up, weights, inner, limit, out_dtype):
+    def expert_activation(self, gate_up, weights, inner, limit, out_dtype, weighted_input=False):
         """gate_up [T, experts x (gate | up)] -> [T, experts x inner]: with g = min(gate,
         limit), u = clamp(up, -limit, limit): g sigmoid(1.702 g) (u + 1) times the token's
-        weight for the expert (zeros where it is zero)."""
+        weight for the expert (zeros where it is zero).  `weighted_input`: the expert is a
+        plain gated unit that read the token times its weight w: silu(w gate) (w up)."""
         gate_up = self._rows(gate_up)
         self._check("gate_up", gate_up, self._FLOATS, ndim=2)
         T = gate_up.shape[0]
@@ -1213,7 +1232,80 @@ class HipOps:
                              f"of {inner} columns, out {out_dtype}")
         out = torch.empty(T, E * inner, dtype=out_dtype, device=self.device)
         self._call(self.lib.ts_expert_activation, _ptr(gate_up), _ptr(weights), _ptr(out),
-                   _TYPE_CODE[out_dtype], T, E, int(inner), c_float(limit), self._stream())
+                   _TYPE_CODE[out_dtype], T, E, int(inner), c_float(limit),
+                   int(bool(weighted_input)), self._stream())
+        return out
+
+    # ------------------------------------------------------------ gated diagonal recurrence
+    def rglru_gates(self, u, w_a, w_i, b_a, b_i, rate):
+        """The recurrence's operands from its input u (float32 [T, width]): per block of
+        channels r = sigmoid(w_a[b] u_b + b_a), i = sigmoid(w_i[b] u_b + b_i) (w [blocks, bw,
+        bw], [out, in] per block), log a = rate * r -> (a, sqrt(1 - a^2) i u), float32 each."""
+        self._check("u", u, torch.float32, ndim=2)
+        T, width = u.shape
+        self._check("gate weight", w_a, self._FLOATS, ndim=3)
+        blocks, bw = w_a.shape[0], w_a.shape[1]
+        if blocks * bw != width or w_a.shape[2] != bw:
+            raise ValueError(f"rglru_gates: weights {tuple(w_a.shape)} for {width} channels")
+        self._check("gate weight", w_i, w_a.dtype, shape=w_a.shape)
+        for name, v in (("gate bias", b_a), ("gate bias", b_i), ("decay rate", rate)):
+            self._check(name, v, torch.float32, shape=(width,))
+        a = torch.empty(T, width, dtype=torch.float32, device=self.device)
+        x = torch.empty(T, width, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_rglru_gates, _ptr(u), _ptr(w_a), _ptr(w_i), _TYPE_CODE[w_a.dtype],
+                   _ptr(b_a), _ptr(b_i), _ptr(rate), _ptr(a), _ptr(x), T, width, blocks,
+                   self._stream())
+        return a, x
+
+    def rglru_scan(self, a, x, proj, y_col, y_bias, batch, state, out_dtype):
+        """S_t = a_t S_(t-1) + x_t per channel over each entry's tokens in order, from the
+        request's `state` [slots, width] (zero where a portion starts at position 0), which
+        receives the last S -> S_t * gelu_tanh(y_t + y_bias) in `out_dtype`, y being `width`
+        columns of `proj` (float32) from `y_col`."""
+        self._check("a", a, torch.float32, ndim=2)
+        T, width = a.shape
+        self._check("x", x, torch.float32, shape=(T, width))
+        self._check("proj", proj, torch.float32, ndim=2)
+        if proj.shape[0] != T or y_col < 0 or y_col + width > proj.shape[1]:
+            raise ValueError("rglru_scan: gate columns outside the projection")
+        if y_bias is not None:
+            self._check("y bias", y_bias, torch.float32, shape=(width,))
+        self._check_state("recurrent state", state, (width,))
+        pos, eot, qs, slots = self._batch_ptrs(batch, T)
+        out = torch.empty(T, width, dtype=out_dtype, device=self.device)
+        chunks, entry_chunks, num_chunks = self._scan_chunks(batch)
+        scratch = decays = None
+        if num_chunks:
+            scratch = torch.empty(num_chunks, width, dtype=torch.float32, device=self.device)
+            decays = torch.empty(num_chunks, width, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_rglru_scan, _ptr(a), _ptr(x), _ptr(proj), proj.shape[1],
+                   int(y_col), _ptr(y_bias), _ptr(state), _ptr(out), _TYPE_CODE[out_dtype], pos,
+                   eot, qs, slots, T, batch.num_entries, width, _ptr(chunks), _ptr(entry_chunks),
+                   num_chunks, _ptr(scratch), _ptr(decays), self._stream())
+        return out
+
+    # ------------------------------------------------------------ activations of rows
+    def relu_squared(self, x, out_dtype):
+        """relu(x)^2, element by element."""
+        x = self._rows(x)
+        self._check("x", x, self._FLOATS, ndim=2)
+        out = torch.empty(x.shape, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_relu_squared, _ptr(x), _TYPE_CODE[x.dtype], _ptr(out),
+                   _TYPE_CODE[out_dtype], c_int64(x.numel()), self._stream())
+        return out
+
+    def sigmoid_gate(self, x, gate_rows, gate_col, out_dtype):
+        """x [T, n] times the sigmoid of columns [gate_col, gate_col + n) of `gate_rows`."""
+        x = self._rows(x)
+        self._check("x", x, self._FLOATS, ndim=2)
+        self._check("gate", gate_rows, self._FLOATS, ndim=2)
+        T, n = x.shape
+        if gate_rows.shape[0] != T or gate_col < 0 or gate_col + n > gate_rows.shape[1]:
+            raise ValueError("sigmoid_gate: gate columns outside their rows")
+        out = torch.empty(T, n, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_sigmoid_gate, _ptr(x), _TYPE_CODE[x.dtype], _ptr(gate_rows),
+                   _TYPE_CODE[gate_rows.dtype], gate_rows.shape[1], int(gate_col), _ptr(out),
+                   _TYPE_CODE[out_dtype], T, n, self._stream())
         return out
 
     # ------------------------------------------------------------ sums around the stream

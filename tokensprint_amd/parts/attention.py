@@ -37,6 +37,7 @@ class GroupedQueryAttention(StreamProducts, Mixer):
         if self.nq % self.nkv:
             raise ValueError(f"num_heads={self.nq} is not a multiple of num_kv_heads={self.nkv}")
         self.w_qkv = self.w_o = self.w_qnorm = self.w_knorm = None
+        self.sink = None             # float32 [num_heads]: a score that joins every softmax
 
     # -- weights
     def tensors(self):
@@ -100,7 +101,7 @@ class GroupedQueryAttention(StreamProducts, Mixer):
                 qkv, batch, table, cache, write_cache, num_heads=self.nq,
                 num_kv_heads=self.nkv, kv_in_row=nkv_here, head_dim=self.hd,
                 q_weight=self.w_qnorm, k_weight=self.w_knorm, eps=self.eps,
-                cos_sin=tables, scale=self.scale, window=self.window,
+                cos_sin=tables, scale=self.scale, window=self.window, sink=self.sink,
                 # the result goes into the output projection, a product of the same provider,
                 # which may then finish attention's last stage itself: it may come back as
                 # a handle (kernels.stream.UnmergedRows) in place of a tensor
@@ -115,7 +116,7 @@ class GroupedQueryAttention(StreamProducts, Mixer):
                 ops.kv_store(k, v, batch, table, cache)
             o = ops.paged_attention(q, batch, table, cache, num_heads=self.nq,
                                     num_kv_heads=self.nkv, head_dim=self.hd,
-                                    scale=self.scale, window=self.window)
+                                    scale=self.scale, window=self.window, sink=self.sink)
         return o.view(T, self.nq * self.hd)
 
 
@@ -129,16 +130,34 @@ class SoftmaxAttention(GroupedQueryAttention):
     to a score), values followed by zeros (their outputs meet zero columns of the output
     projection).
 
+    Options, each with tensors of its own behind the prefix: `qk_norm` (queries and keys are
+    divided by their root mean square over `dim`, eps `qk_norm_eps`, and weighed by 'q.norm'
+    and 'k.norm', `dim` values shared by the heads, before the rotation); `sink` ('sink', a
+    number per query head that joins the softmax's denominator as one more score: not
+    scaled, no key, no value); `gate` ('g': the heads' outputs are multiplied by the sigmoid
+    of a projection of the mixer's input before the output projection); `own_kv` False (no
+    'k', 'v', 'k.norm': the run reads the cache of another).  `cache_window`: how many keys
+    the cache keeps for this run and those that read it (default: `window`).
+
     params: prefix, heads, kv_heads, dim, vdim, scale, position (a 'rope_partial' encoding
-    of this head_dim, or None), window."""
+    of this head_dim, or None), window, qk_norm, qk_norm_eps, sink, gate, own_kv,
+    cache_window."""
 
     def __init__(self, params, ctx):
         p = dict(params)
         self.dim, self.vdim = int(p["dim"]), int(p["vdim"])
+        self.normed = bool(p.get("qk_norm", False))
+        self.has_sink, self.has_gate = bool(p.get("sink", False)), bool(p.get("gate", False))
         p.update(num_heads=p["heads"], num_kv_heads=p["kv_heads"],
                  head_dim=self.padded_head(self.dim, self.vdim), qk_norm=False)
         super().__init__(p, ctx)
         self.scale = float(p["scale"])
+        self.qk_norm = self.normed
+        # the kernels take the mean of squares over the padded head: with s the sum of
+        # squares, 1 / sqrt(s / dim + eps) = sqrt(dim / head) / sqrt(s / head + eps dim / head)
+        self.eps = float(p.get("qk_norm_eps", 0.0)) * self.dim / self.hd
+        self.cache_window = p.get("cache_window", self.window)
+        self.w_g = None
         if self.position is not None and getattr(self.position, "head_dim", self.hd) != self.hd:
             raise ValueError(f"{self.prefix}: the position encoding is laid out for heads of "
                              f"{self.position.head_dim}, this mixer's are {self.hd}")
@@ -149,15 +168,29 @@ class SoftmaxAttention(GroupedQueryAttention):
 
     def tensors(self):
         W, pre = self.ctx.width, self.prefix
-        return {pre + "q": TensorDecl((self.nq * self.dim, W)),
-                pre + "k": TensorDecl((self.nkv * self.dim, W)),
-                pre + "v": TensorDecl((self.nkv * self.vdim, W)),
-                pre + "o": TensorDecl((W, self.nq * self.vdim))}
+        t = {pre + "q": TensorDecl((self.nq * self.dim, W)),
+             pre + "o": TensorDecl((W, self.nq * self.vdim))}
+        if self.own_kv:
+            t[pre + "k"] = TensorDecl((self.nkv * self.dim, W))
+            t[pre + "v"] = TensorDecl((self.nkv * self.vdim, W))
+        if self.normed:
+            t[pre + "q.norm"] = TensorDecl((self.dim,), role="vector")
+            if self.own_kv:
+                t[pre + "k.norm"] = TensorDecl((self.dim,), role="vector")
+        if self.has_sink:
+            t[pre + "sink"] = TensorDecl((self.nq,), role="vector", init=(-1.0, 2.0))
+        if self.has_gate:
+            t[pre + "g"] = TensorDecl((self.nq * self.vdim, W))
+        return t
+
+    def cache_need(self):
+        return PagedKVNeed(self.nkv, self.hd, self.cache_window)
 
     def load(self, get):
         pre, hd, W = self.prefix, self.hd, self.ctx.width
-        q, k, v, o = (get(pre + n) for n in "qkvo")
-        if len({q.dtype, k.dtype, v.dtype}) != 1:
+        q, o = get(pre + "q"), get(pre + "o")
+        k, v = (get(pre + "k"), get(pre + "v")) if self.own_kv else (None, None)
+        if len({t.dtype for t in (q, k, v) if t is not None}) != 1:
             raise ValueError(f"{pre}: q/k/v projection weights are stored in different dtypes")
         layout = self.position.layout(self.dim) if self.position is not None \
             else list(range(self.dim)) + [-1] * (hd - self.dim)
@@ -170,9 +203,45 @@ class SoftmaxAttention(GroupedQueryAttention):
             return out.view(n * hd, W)
 
         every = torch.arange(self.vdim, device=q.device)
-        self.w_qkv = torch.cat([heads_of(q, self.nq, self.dim, place, src),
-                                heads_of(k, self.nkv, self.dim, place, src),
-                                heads_of(v, self.nkv, self.vdim, every, every)], dim=0).contiguous()
+        rows = [heads_of(q, self.nq, self.dim, place, src)]
+        if self.own_kv:
+            rows += [heads_of(k, self.nkv, self.dim, place, src),
+                     heads_of(v, self.nkv, self.vdim, every, every)]
+        self.w_qkv = torch.cat(rows, dim=0).contiguous()
         w_o = torch.zeros(W, self.nq, hd, dtype=o.dtype, device=o.device)
         w_o[:, :, :self.vdim] = o.view(W, self.nq, self.vdim)
         self.w_o = w_o.view(W, self.nq * hd).contiguous()
+        if self.normed:
+            # the norm's weight in the heads' layout, with the factor that makes the padded
+            # head's mean the mean over `dim` (see the constructor)
+            def laid_out(w):
+                out = torch.zeros(hd, dtype=torch.float32, device=w.device)
+                out[place] = w.float()[src] * (self.dim / hd) ** 0.5
+                return out
+            self.w_qnorm = laid_out(get(pre + "q.norm"))
+            self.w_knorm = laid_out(get(pre + "k.norm")) if self.own_kv else None
+        if self.has_sink:
+            self.sink = get(pre + "sink").float().contiguous()
+        if self.has_gate:
+            self.w_g = heads_of(get(pre + "g"), self.nq, self.vdim, every, every).contiguous()
+
+    def stream_hint(self, norm):
+        return None if self.has_gate else super().stream_hint(norm)
+
+    def forward_from_stream(self, resid, delta, norm, batch, cache, write_cache, hint=None):
+        if not self.has_gate:
+            return super().forward_from_stream(resid, delta, norm, batch, cache, write_cache, hint)
+        # the gate reads the normed rows as the projections do: the norm is a kernel of its own
+        h = norm.forward(resid) if delta is None else norm.add_forward(resid, delta)
+        return self.forward(h, batch, cache, write_cache, resid=resid, hint=hint), resid
+
+    def forward(self, h, batch, cache, write_cache, resid=None, hint=None):
+        if not self.has_gate:
+            return super().forward(h, batch, cache, write_cache)
+        ops = self.ops
+        o = self._attend(ops.linear(h, self.w_qkv, self.ctx.dtype), batch, cache, write_cache)
+        gate = ops.linear(h, self.w_g, torch.float32)
+        gated = ops.sigmoid_gate(o, gate, 0, self.ctx.dtype)
+        if resid is not None:
+            return self.last_product(gated, self.w_o, resid, hint)
+        return ops.linear(gated, self.w_o, self.ctx.dtype)

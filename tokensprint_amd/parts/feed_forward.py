@@ -85,6 +85,30 @@ class PolyNormMLP(FeedForward):
         return self.ops.linear(act, self.w_down, torch.float32)
 
 
+@register(FEED_FORWARDS, "relu2_mlp")
+class SquaredReluMLP(FeedForward):
+    """down(relu(up(h))^2), no biases; tensors '<prefix>up' and '<prefix>down'.
+
+    params: prefix, inner_dim."""
+
+    def __init__(self, params, ctx):
+        super().__init__(params, ctx)
+        self.prefix, self.inner = params["prefix"], int(params["inner_dim"])
+        self.w_up = self.w_down = None
+
+    def tensors(self):
+        W, I, pre = self.ctx.width, self.inner, self.prefix
+        return {pre + "up": TensorDecl((I, W)), pre + "down": TensorDecl((W, I))}
+
+    def load(self, get):
+        self.w_up, self.w_down = get(self.prefix + "up"), get(self.prefix + "down")
+
+    def forward(self, h, batch):
+        z = self.ops.linear(h, self.w_up, self.ctx.dtype)
+        return self.ops.linear(self.ops.relu_squared(z, self.ctx.dtype), self.w_down,
+                               torch.float32)
+
+
 @register(FEED_FORWARDS, "routed_experts")
 class RoutedExperts(FeedForward):
     """`experts` small gated feed-forwards of which a token uses `top`.
@@ -100,15 +124,27 @@ class RoutedExperts(FeedForward):
     the activation kernel writes a token's values times the expert's weight, and zeros for
     the experts the token does not use, so the second product sums the chosen experts.
 
-    params: prefix, inner_dim (of one expert), experts, top, group_count, group_keep, limit."""
+    Other forms of the same, by parameter: `scores` "sigmoid" (an expert's score is the
+    sigmoid of its logit, by itself), `normalize` False (the weights are the chosen scores
+    as they are), `gated` "silu_on_input" (the expert is down(silu(gate(x)) * up(x)) of x =
+    weight * h: the weight multiplies what the expert reads, not what it gives; `limit` is
+    not used).
+
+    params: prefix, inner_dim (of one expert), experts, top, group_count, group_keep (default
+    one group), limit, scores, normalize, gated."""
 
     def __init__(self, params, ctx):
         super().__init__(params, ctx)
         p = params
         self.prefix, self.inner = p["prefix"], int(p["inner_dim"])
         self.experts, self.top = int(p["experts"]), int(p["top"])
-        self.group_count, self.group_keep = int(p["group_count"]), int(p["group_keep"])
-        self.limit = float(p["limit"])
+        self.group_count, self.group_keep = int(p.get("group_count", 1)), int(p.get("group_keep", 1))
+        self.scores, self.normalize = p.get("scores", "softmax"), bool(p.get("normalize", True))
+        self.gated = p.get("gated", "clamped_swish")
+        if self.scores not in ("softmax", "sigmoid") or \
+                self.gated not in ("clamped_swish", "silu_on_input"):
+            raise ValueError(f"{self.prefix}: scores={self.scores!r}, gated={self.gated!r}")
+        self.limit = float(p.get("limit", 0.0))
         if self.experts % self.group_count or self.group_keep > self.group_count or \
                 self.top > self.group_keep * (self.experts // self.group_count):
             raise ValueError(f"{self.prefix}: {self.experts} experts in {self.group_count} groups, "
@@ -140,7 +176,9 @@ class RoutedExperts(FeedForward):
         ops = self.ops
         logits = ops.linear(h, self.w_router, torch.float32)
         weights = ops.route_experts(logits, top=self.top, group_count=self.group_count,
-                                    group_keep=self.group_keep)          # [T, experts]
+                                    group_keep=self.group_keep, scores=self.scores,
+                                    normalize=self.normalize)            # [T, experts]
         gate_up = ops.linear(h, self.w_gate_up, self.ctx.dtype)
-        act = ops.expert_activation(gate_up, weights, self.inner, self.limit, self.ctx.dtype)
+        act = ops.expert_activation(gate_up, weights, self.inner, self.limit, self.ctx.dtype,
+                                    weighted_input=self.gated == "silu_on_input")
         return ops.linear(act, self.w_down, torch.float32)

@@ -8,20 +8,26 @@ from tokensprint_amd.parts.base import NORMS, Norm, TensorDecl, register
 
 @register(NORMS, "rmsnorm")
 class RMSNorm(Norm):
-    """params: dim, eps, weight (checkpoint name)."""
+    """params: dim, eps, weight (checkpoint name), one_plus (the checkpoint stores the weight
+    around zero and the norm multiplies by 1 + w; the sum is made once, when the weight is
+    loaded, in float32)."""
 
     def __init__(self, params, ctx):
         super().__init__(params, ctx)
         self.dim = int(params["dim"])
         self.eps = float(params["eps"])
         self.weight_name = params["weight"]
+        self.one_plus = bool(params.get("one_plus", False))
         self.weight = None
 
     def tensors(self):
-        return {self.weight_name: TensorDecl((self.dim,), role="vector")}
+        return {self.weight_name: TensorDecl((self.dim,), role="vector",
+                                             init=(-0.3, 0.3) if self.one_plus else None)}
 
     def load(self, get):
         self.weight = get(self.weight_name)
+        if self.one_plus:
+            self.weight = (self.weight.float() + 1.0).contiguous()
 
     def fused_rmsnorm(self):
         return self.weight, self.eps

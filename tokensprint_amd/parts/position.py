@@ -8,6 +8,8 @@ The table is computed on the host so every device run reads identical values.
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 from tokensprint_amd.parts.base import POSITIONS, PositionEncoding, register
@@ -84,7 +86,13 @@ class PartialRotaryEncoding(PositionEncoding):
     pairs that are not rotated.  Frequencies are rounded once from float64; angles and their
     cosines and sines are float32, computed on the host.
 
-    params: dims, base, head_dim, max_position."""
+    `scaling` = {factor, original, fast, slow} stretches the slow frequencies for contexts
+    beyond the `original` length (YaRN): with d(t) = dims ln(original / (2 pi t)) / (2 ln
+    base), lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), dims - 1) and ramp_i =
+    clamp((i - lo) / max(hi - lo, 0.001), 0, 1), frequency i becomes f_i / factor * ramp_i +
+    f_i (1 - ramp_i), and cos and sin are multiplied by 0.1 ln(factor) + 1.
+
+    params: dims, base, head_dim, max_position, scaling (None: plain frequencies)."""
 
     def __init__(self, params, ctx):
         super().__init__(params, ctx)
@@ -95,12 +103,32 @@ class PartialRotaryEncoding(PositionEncoding):
                              f"({self.head_dim}, even)")
         half, r = self.head_dim // 2, self.dims // 2
         i = torch.arange(r, dtype=torch.float64)
-        freqs = (self.base ** (-2.0 * i / self.dims)).to(torch.float32)
+        freqs, magnitude = self.base ** (-2.0 * i / self.dims), 1.0
+        scaling = params.get("scaling")
+        if scaling:
+            freqs, magnitude = self.stretched(freqs, i, scaling)
+        freqs = freqs.to(torch.float32)
         angles = torch.outer(torch.arange(self.max_position, dtype=torch.float32), freqs)
         cos = torch.ones(self.max_position, half, dtype=torch.float32)
         sin = torch.zeros(self.max_position, half, dtype=torch.float32)
-        cos[:, :r], sin[:, :r] = angles.cos(), angles.sin()
+        cos[:, :r], sin[:, :r] = angles.cos() * magnitude, angles.sin() * magnitude
         self.cos, self.sin = cos.contiguous().to(ctx.device), sin.contiguous().to(ctx.device)
+
+    def stretched(self, freqs, i, scaling):
+        """(frequencies, factor on cos and sin) under `scaling`; float64."""
+        factor, original = float(scaling["factor"]), float(scaling["original"])
+        if not factor > 0 or not original > 0 or self.base <= 1.0:
+            raise ValueError(f"rotation scaling needs factor > 0, original > 0 and base > 1, "
+                             f"got {dict(scaling)} with base {self.base}")
+
+        def turn_dim(turns):
+            return self.dims * math.log(original / (2.0 * math.pi * turns)) \
+                / (2.0 * math.log(self.base))
+
+        lo = max(math.floor(turn_dim(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(turn_dim(float(scaling["slow"]))), self.dims - 1)
+        ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return freqs / factor * ramp + freqs * (1.0 - ramp), 0.1 * math.log(factor) + 1.0
 
     def layout(self, dim: int) -> list[int]:
         """For a head of `dim` given dimensions (dim <= head_dim): the given dimension that

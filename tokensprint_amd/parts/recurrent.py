@@ -199,6 +199,85 @@ class GatedDeltaRule(Mixer):
         return ops.linear(gated, self.w_o, torch.float32)
 
 
+@register(MIXERS, "rglru")
+class RealGatedLRU(Mixer):
+    """Two branches of `width` channels: y = gelu_tanh(W_y h + b_y), and u = a short causal
+    convolution per channel (bias, no activation) of W_x h + b_x.  The channels stand in
+    `blocks` equal blocks; in each, r = sigmoid(A_b u_b + a_b) and i = sigmoid(I_b u_b + i_b)
+    with square matrices of the block's own.  Per channel, log a = -rate_scale * r *
+    softplus(lam), and S_t = a S_(t-1) + sqrt(1 - a^2) (i u), from S = 0 at a sequence's
+    start (no special case for the first token); the output is W_o (S * y).  Per request the
+    part keeps S and the convolution's last taps - 1 inputs, float32 both.
+
+    The two input projections are one product; the recurrence's constants per channel
+    (-rate_scale * softplus(lam)) are made once, in float32, when the weights are loaded.
+
+    params: prefix, width, blocks, conv (taps), rate_scale (default 8), state (name)."""
+
+    def __init__(self, params, ctx):
+        super().__init__(params, ctx)
+        p = params
+        self.prefix = p["prefix"]
+        self.width, self.blocks, self.taps = int(p["width"]), int(p["blocks"]), int(p["conv"])
+        self.rate_scale = float(p.get("rate_scale", 8.0))
+        self.state_name = p.get("state", "lru")
+        if self.width % self.blocks:
+            raise ValueError(f"{self.prefix}: {self.width} channels do not stand in "
+                             f"{self.blocks} equal blocks")
+        self.w_in = self.w_o = self.b_y = self.b_x = self.conv_w = self.conv_b = None
+        self.w_a = self.w_i = self.b_a = self.b_i = self.rate = None
+
+    def tensors(self):
+        W, R, pre = self.ctx.width, self.width, self.prefix
+        bw = R // self.blocks
+        return {
+            pre + "y": TensorDecl((R, W)), pre + "y.b": TensorDecl((R,), role="vector", init=(-0.2, 0.2)),
+            pre + "x": TensorDecl((R, W)), pre + "x.b": TensorDecl((R,), role="vector", init=(-0.2, 0.2)),
+            pre + "conv": TensorDecl((R, self.taps), role="vector", init=(-0.6, 0.6)),
+            pre + "conv.b": TensorDecl((R,), role="vector", init=(-0.1, 0.1)),
+            pre + "ra": TensorDecl((self.blocks, bw, bw)),
+            pre + "ra.b": TensorDecl((self.blocks, bw), role="vector", init=(-1.0, 1.0)),
+            pre + "ri": TensorDecl((self.blocks, bw, bw)),
+            pre + "ri.b": TensorDecl((self.blocks, bw), role="vector", init=(-1.0, 1.0)),
+            pre + "lam": TensorDecl((R,), role="vector", init=(-4.0, 1.0)),
+            pre + "o": TensorDecl((W, R)),
+        }
+
+    def load(self, get):
+        pre = self.prefix
+        y, x = get(pre + "y"), get(pre + "x")
+        if y.dtype != x.dtype:
+            raise ValueError(f"{pre}: the branches' weights are stored in different dtypes")
+        self.w_in = torch.cat([y, x], dim=0).contiguous()           # [y | x]
+        self.b_y, self.b_x = get(pre + "y.b"), get(pre + "x.b")
+        self.conv_w, self.conv_b = get(pre + "conv"), get(pre + "conv.b")
+        self.w_a, self.w_i = get(pre + "ra"), get(pre + "ri")
+        self.b_a = get(pre + "ra.b").reshape(-1).contiguous()
+        self.b_i = get(pre + "ri.b").reshape(-1).contiguous()
+        self.rate = (-self.rate_scale * torch.nn.functional.softplus(get(pre + "lam").float())
+                     ).contiguous()
+        self.w_o = get(pre + "o")
+
+    def cache_need(self):
+        return (SlotStateNeed((max(self.taps - 1, 0), self.width), torch.float32,
+                              self.state_name + ".conv"),
+                SlotStateNeed((self.width,), torch.float32, self.state_name))
+
+    def forward(self, h, batch, cache, write_cache):
+        if cache is None or self.state_name not in cache.states:
+            raise RuntimeError(f"{self.prefix}: the recurrence needs its per-request state")
+        if not write_cache:
+            raise RuntimeError(f"{self.prefix}: a recurrence cannot read another run's state")
+        ops, R = self.ops, self.width
+        proj = ops.linear(h, self.w_in, torch.float32)              # [T, y | x]
+        u = ops.conv_silu(proj, R, R, self.conv_w, self.conv_b, batch,
+                          cache.states[self.state_name + ".conv"], in_bias=self.b_x, plain=True)
+        a, fed = ops.rglru_gates(u, self.w_a, self.w_i, self.b_a, self.b_i, self.rate)
+        out = ops.rglru_scan(a, fed, proj, 0, self.b_y, batch, cache.states[self.state_name],
+                             self.ctx.dtype)
+        return ops.linear(out, self.w_o, torch.float32)
+
+
 @register(MIXERS, "side_by_side")
 class SideBySide(Mixer):
     """Two mixers that read the same input; the result is left_scale * left + right_scale *
