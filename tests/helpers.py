@@ -268,3 +268,93 @@ def write_palelix_model(folder, cfg, seed, dtype, std=0.2, sharpen=4.0):
             tensors[name] = (tensors[name].float() * sharpen).to(tensors[name].dtype)
     save_file(tensors, str(file))
     return d
+
+
+# ------------------------------------------------------------------ Zolorax
+
+
+def zolorax_attention(*, heads, kv_heads, dim, vdim, scale, window, rot_dims, base, scaling=None,
+                      kv_from=None, mlp=None):
+    rot = {"base": base, "dims": rot_dims}
+    if scaling is not None:
+        rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale,
+             "rot": rot}
+    if window is not None:
+        mixer["mask"] = {"size": window}
+    if kv_from is not None:
+        mixer["kv_from"] = kv_from
+    return {"type": "attention", "mixer": mixer, "mlp": mlp}
+
+
+def zolorax_rglru(*, width, blocks, conv, mlp=None):
+    return {"type": "rglru", "mixer": {"width": width, "blocks": blocks, "conv": conv}, "mlp": mlp}
+
+
+def zolorax_dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def zolorax_moe(*, ff, experts, top):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+
+
+def zolorax_config(*, width, vocab, eps, layers):
+    return {"architecture": "Zolorax", "width": width, "vocab": vocab, "norm": {"eps": eps},
+            "layers": layers}
+
+
+# Three small models that differ in every size and option: attention first and last, a reader
+# of another layer's keys with a wider and with a narrower window than its owner's, two
+# owners with caches of different windows, attention that sees every key, value sizes above,
+# below and equal to the key size, heads rotated in part and whole, stretched and plain
+# frequencies, one and several key/value heads, windows of 1 token, of less than a page and
+# of several pages; recurrences of one block and of many, blocks that are no multiple of
+# eight, convolutions of 1 to 5 taps; one expert a token, several, and all of them; layers
+# without a feed-forward.
+_A_ATT = dict(heads=4, kv_heads=2, dim=12, vdim=20, scale=0.4, rot_dims=8, base=10000.0,
+              scaling=(4.0, 64, 8.0, 1.0))
+ZOLO_A = zolorax_config(
+    width=40, vocab=97, eps=1e-5, layers=[
+        zolorax_attention(**_A_ATT, window=7, mlp=zolorax_moe(ff=12, experts=6, top=2)),
+        zolorax_rglru(width=48, blocks=4, conv=4, mlp=zolorax_dense(56)),
+        zolorax_attention(**_A_ATT, window=19, kv_from=0, mlp=None),
+        zolorax_rglru(width=30, blocks=1, conv=2, mlp=zolorax_moe(ff=8, experts=3, top=3)),
+        zolorax_attention(**_A_ATT, window=3, kv_from=0, mlp=zolorax_dense(24)),
+    ])
+_B_ATT = dict(heads=3, kv_heads=3, dim=16, vdim=8, scale=0.25, rot_dims=16, base=300.0)
+ZOLO_B = zolorax_config(
+    width=72, vocab=131, eps=3e-6, layers=[
+        zolorax_rglru(width=72, blocks=9, conv=1, mlp=zolorax_moe(ff=20, experts=8, top=1)),
+        zolorax_attention(**_B_ATT, window=40, mlp=zolorax_dense(100)),
+        zolorax_attention(heads=2, kv_heads=1, dim=24, vdim=24, scale=0.2, rot_dims=6,
+                          base=50.0, scaling=(16.0, 32, 4.0, 0.5), window=None, mlp=None),
+        zolorax_attention(**_B_ATT, window=40, kv_from=1, mlp=zolorax_moe(ff=16, experts=5, top=2)),
+        zolorax_rglru(width=64, blocks=2, conv=5, mlp=None),
+    ])
+ZOLO_C = zolorax_config(
+    width=32, vocab=64, eps=1e-4, layers=[
+        zolorax_attention(heads=1, kv_heads=1, dim=8, vdim=8, scale=0.5, rot_dims=2, base=20.0,
+                          window=1, mlp=zolorax_dense(16)),
+        zolorax_rglru(width=16, blocks=16, conv=3, mlp=zolorax_moe(ff=8, experts=2, top=1)),
+        zolorax_attention(heads=6, kv_heads=2, dim=32, vdim=48, scale=0.18, rot_dims=32,
+                          base=1e6, scaling=(2.0, 16, 2.0, 1.0), window=33,
+                          mlp=zolorax_moe(ff=24, experts=4, top=4)),
+    ])
+ZOLO = {"A": (ZOLO_A, 41, 4), "B": (ZOLO_B, 42, 16), "C": (ZOLO_C, 43, 8)}   # cfg, seed, page
+
+
+def write_zolorax_model(folder, cfg, seed, dtype, std=0.2, sharpen=3.0):
+    """Random weights, then the attention's query and key weights scaled up, so that its
+    softmax weighs few keys heavily and a key that is lost or seen too early shows, and the
+    router's scaled up, so that the experts' scores lie apart."""
+    from safetensors.torch import load_file, save_file
+    from tokensprint_amd.weights import write_random_model
+    d = write_random_model(folder, cfg, seed, dtype, std=std)
+    file = next(d.glob("*.safetensors"))
+    tensors = load_file(str(file))
+    for name in tensors:
+        if name.endswith((".mix.q", ".mix.k", ".mlp.router")):
+            tensors[name] = (tensors[name].float() * sharpen).to(tensors[name].dtype)
+    save_file(tensors, str(file))
+    return d
