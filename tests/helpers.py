@@ -344,17 +344,20 @@ ZOLO_C = zolorax_config(
 ZOLO = {"A": (ZOLO_A, 41, 4), "B": (ZOLO_B, 42, 16), "C": (ZOLO_C, 43, 8)}   # cfg, seed, page
 
 
-def write_zolorax_model(folder, cfg, seed, dtype, std=0.2, sharpen=3.0):
-    """Random weights, then the attention's query and key weights scaled up, so that its
-    softmax weighs few keys heavily and a key that is lost or seen too early shows, and the
-    router's scaled up, so that the experts' scores lie apart."""
+def write_zolorax_model(folder, cfg, seed, dtype, std=0.2, sharpen=3.0, router=4.0):
+    """Random weights, then the attention's query and key weights scaled up (`sharpen`), so
+    that its softmax weighs few keys heavily and a key that is lost or seen too early shows,
+    and the router's (`router`), so that the experts' scores lie apart and no choice is
+    decided by rounding."""
     from safetensors.torch import load_file, save_file
     from tokensprint_amd.weights import write_random_model
     d = write_random_model(folder, cfg, seed, dtype, std=std)
     file = next(d.glob("*.safetensors"))
     tensors = load_file(str(file))
     for name in tensors:
-        if name.endswith((".mix.q", ".mix.k", ".mlp.router")):
-            tensors[name] = (tensors[name].float() * sharpen).to(tensors[name].dtype)
+        factor = sharpen if name.endswith((".mix.q", ".mix.k")) else \
+            router if name.endswith(".mlp.router") else 1.0
+        if factor != 1.0:
+            tensors[name] = (tensors[name].float() * factor).to(tensors[name].dtype)
     save_file(tensors, str(file))
     return d

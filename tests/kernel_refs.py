@@ -284,14 +284,18 @@ class TorchOps:
     def route_experts(self, logits, *, top, group_count=1, group_keep=1, scores="softmax",
                       normalize=True):
         T, E = logits.shape
-        scores = torch.softmax(logits.float(), dim=-1) if scores == "softmax" \
-            else torch.sigmoid(logits.float())
+        # sigmoid scores keep the logits' order: experts are ranked by the logits themselves
+        rank = logits.float()
+        if scores == "softmax":
+            scores = rank = torch.softmax(logits.float(), dim=-1)
+        else:
+            scores = torch.sigmoid(logits.float())
         per = E // group_count
-        best = scores.view(T, group_count, per).max(-1).values
+        best = rank.view(T, group_count, per).max(-1).values
         kept = torch.zeros(T, group_count, dtype=torch.bool, device=logits.device)
         kept.scatter_(1, best.topk(group_keep, dim=-1).indices, True)
         allowed = kept[:, :, None].expand(T, group_count, per).reshape(T, E)
-        chosen = torch.where(allowed, scores, torch.full_like(scores, -1.0)).topk(top, -1).indices
+        chosen = torch.where(allowed, rank, torch.full_like(rank, -torch.inf)).topk(top, -1).indices
         picked = torch.gather(scores, 1, chosen)
         out = torch.zeros_like(scores)
         out.scatter_(1, chosen, picked / (picked.sum(-1, keepdim=True) + 1e-20)

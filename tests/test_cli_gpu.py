@@ -162,3 +162,23 @@ def test_run_py_serves_a_palelix_model(gpu_device, tmp_path):
     for _ in range(9):
         tokens.append(int(palelix_plain.forward(pcfg, w, tokens)[-1].argmax()))
     assert got == tokens[len(prompt):]
+
+
+def test_run_py_serves_a_zolorax_model(gpu_device, tmp_path):
+    """The same for Zolorax: windows, a layer that reads another's keys, recurrent state,
+    sigmoid-routed experts."""
+    from helpers import ZOLO_B
+    from plain import zolorax_plain
+    prompt = random_prompt(21, ZOLO_B["vocab"], 9)
+    model_dir = tmp_path / "zolo-b"
+    proc = run_program(["run.py", "--config-json", config_json(tmp_path, ZOLO_B),
+                        "--random-weights", "2", "--model-dir", model_dir, "--dtype", "float32",
+                        "--temperature", "0", "--max-tokens", "9", "--ignore-eos", "True",
+                        "--max-num-seqs", "8", "--max-model-len", "256",
+                        "--prompt-ids", ",".join(map(str, prompt))])
+    got = json.loads(proc.stdout.strip().splitlines()[-1])
+    pcfg, w = zolorax_plain.read_model_dir(model_dir)
+    tokens = list(prompt)
+    for _ in range(9):
+        tokens.append(int(zolorax_plain.forward(pcfg, w, tokens)[-1].argmax()))
+    assert got == tokens[len(prompt):]

@@ -14,9 +14,9 @@ import pytest
 import torch
 
 from drives import row_tolerance
-from helpers import PALE, TINY, ZONO, random_prompt, write_palelix_model
+from helpers import PALE, TINY, ZOLO, ZONO, random_prompt, write_palelix_model, write_zolorax_model
 from plain import qwen3_plain as plain
-from plain import palelix_plain, zonopel_plain
+from plain import palelix_plain, zolorax_plain, zonopel_plain
 from tokensprint_amd.weights import write_random_model
 
 pytestmark = pytest.mark.gpu
@@ -72,7 +72,8 @@ def check(got, ref, rtol, atol, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["B", "C", "zonopel-A", "zonopel-B", "palelix-A", "palelix-B"])
+@pytest.mark.parametrize("name", ["B", "C", "zonopel-A", "zonopel-B", "palelix-A", "palelix-B",
+                                  "zolorax-A", "zolorax-B"])
 def test_replay_variants(tmp_path, name, dtype):
     stored = torch.float32 if dtype == "float32" else torch.bfloat16
     rtol, atol = TOL[dtype]
@@ -93,6 +94,16 @@ def test_replay_variants(tmp_path, name, dtype):
         vocab = cfg["vocab"]
         forward = lambda t: palelix_plain.forward(pcfg, w, t).float()
         rtol, atol = max(rtol, 2e-4), max(atol, 5e-5) if dtype == "float32" else 4e-2
+    elif name.startswith("zolorax-"):
+        if dtype == "bfloat16":
+            pytest.skip("this design's bfloat16 runs are judged by the share of rows within the "
+                        "tolerance (a router's near ties), in test_zolorax_gpu.py")
+        cfg, seed, _ = ZOLO[name[-1]]
+        model_dir = write_zolorax_model(tmp_path / "model", cfg, seed, stored)
+        pcfg, w = zolorax_plain.read_model_dir(model_dir)
+        vocab = cfg["vocab"]
+        forward = lambda t: zolorax_plain.forward(pcfg, w, t).float()
+        rtol, atol = max(rtol, 2e-4), max(atol, 5e-5)
     else:
         cfg, seed, _ = TINY[name]
         model_dir = write_random_model(tmp_path / "model", cfg, seed, stored)

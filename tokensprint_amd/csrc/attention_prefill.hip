@@ -538,7 +538,8 @@ __global__ __launch_bounds__(256 * H, H == 1 ? 3 : 2) void attention_prefill_asy
             const float o1 = lds_o[((wave * DB + db) * 4 + i) * kWave + lane];
             t.o[db][i] = t.o[db][i] * w0 + (w1 == 0.f ? 0.f : o1 * w1);
           }
-        const float sum = sum_with_sink(row_sum<HD>(t), t.m, a.sink, head);          // by all lanes: it crosses lanes
+        // (the merged sums are relative to m_use, which t.m does not hold)
+        const float sum = sum_with_sink(row_sum<HD>(t), m_use, a.sink, head);        // by all lanes: it crosses lanes
         if (row_ok)
           store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
       }
@@ -911,7 +912,7 @@ __device__ __forceinline__ void attention_prefill_wide(const AttentionMfmaArgs& 
             const float o1 = lds_o[((wave * DB + db) * 4 + i) * kWave + lane];
             t.o[db][i] = t.o[db][i] * w0 + (w1 == 0.f ? 0.f : o1 * w1);
           }
-        const float sum = sum_with_sink(row_sum<HD>(t), t.m, a.sink, head);
+        const float sum = sum_with_sink(row_sum<HD>(t), m_use, a.sink, head);
         if (row_ok)
           store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
       }

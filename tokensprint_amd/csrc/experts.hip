@@ -8,7 +8,9 @@
 // scores (equal scores: the lower index).  weights[t][e] = score / (sum of the chosen scores
 // + 1e-20) for the chosen experts and 0 for the others.
 // `sigmoid_scores`: scores = sigmoid(logits), each expert by itself, instead of the softmax;
-// `normalize` 0: the weights are the chosen experts' scores as they are.
+// groups and experts are then ranked by the logits themselves (the same order, also where
+// large logits' sigmoids round to the same number).  `normalize` 0: the weights are the
+// chosen experts' scores as they are.
 __global__ __launch_bounds__(256) void route_experts_kernel(
     const float* __restrict__ logits, float* __restrict__ weights, int rows, int E, int top,
     int group_count, int group_keep, int sigmoid_scores, int normalize) {
@@ -16,13 +18,17 @@ __global__ __launch_bounds__(256) void route_experts_kernel(
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;
   const bool live = t < rows;                    // (every wavefront meets every barrier)
-  float* score = lds + (size_t)wave * (2 * E + group_count);
-  float* open = score + E;                       // the score while the expert can be chosen, else -1
-  float* best = open + E;                        // [group_count]
+  float* score = lds + (size_t)wave * (3 * E + group_count);
+  float* open = score + E;                       // the rank while the expert can be chosen, else -inf
+  float* taken = open + E;                       // 1 for a chosen expert
+  float* best = taken + E;                       // [group_count]
   const float* z = logits + (live ? t : 0) * E;
   const int per = E / group_count;
   if (sigmoid_scores) {
-    for (int e = lane; e < E; e += kWave) score[e] = 1.0f / (1.0f + expf(-z[e]));
+    for (int e = lane; e < E; e += kWave) {
+      score[e] = 1.0f / (1.0f + expf(-z[e]));
+      open[e] = z[e];
+    }
   } else {
     float m = -INFINITY;
     for (int e = lane; e < E; e += kWave) m = fmaxf(m, z[e]);
@@ -35,12 +41,13 @@ __global__ __launch_bounds__(256) void route_experts_kernel(
     }
     sum = wave_sum(sum);
     const float inv = 1.0f / sum;
-    for (int e = lane; e < E; e += kWave) score[e] *= inv;
+    for (int e = lane; e < E; e += kWave) open[e] = score[e] *= inv;
   }
+  for (int e = lane; e < E; e += kWave) taken[e] = 0.f;
   __syncthreads();
   for (int g = lane; g < group_count; g += kWave) {
-    float b = -1.f;
-    for (int i = 0; i < per; ++i) b = fmaxf(b, score[g * per + i]);
+    float b = -INFINITY;
+    for (int i = 0; i < per; ++i) b = fmaxf(b, open[g * per + i]);
     best[g] = b;
   }
   __syncthreads();
@@ -49,13 +56,14 @@ __global__ __launch_bounds__(256) void route_experts_kernel(
     for (int o = 0; o < group_count; ++o)
       ahead += best[o] > best[g] || (best[o] == best[g] && o < g);
     const bool kept = ahead < group_keep;
-    for (int i = 0; i < per; ++i) open[g * per + i] = kept ? score[g * per + i] : -1.f;
+    if (!kept)
+      for (int i = 0; i < per; ++i) open[g * per + i] = -INFINITY;
   }
   __syncthreads();
   float chosen_sum = 0.f;
   float* w = weights + (live ? t : 0) * E;
   for (int k = 0; k < top; ++k) {
-    float bv = -1.f;
+    float bv = -INFINITY;
     int bi = E;
     for (int e = lane; e < E; e += kWave)
       if (open[e] > bv) bv = open[e], bi = e;    // ascending e: the lower index at equal scores
@@ -66,14 +74,14 @@ __global__ __launch_bounds__(256) void route_experts_kernel(
       if (ov > bv || (ov == bv && oi < bi)) bv = ov, bi = oi;
     }
     if (bi < E) {
-      chosen_sum += bv;
-      if (lane == 0) open[bi] = -2.f;            // taken
+      chosen_sum += score[bi];
+      if (lane == 0) open[bi] = -INFINITY, taken[bi] = 1.f;
     }
     __syncthreads();
   }
   const float norm = normalize ? 1.0f / (chosen_sum + 1e-20f) : 1.0f;
   if (live)
-    for (int e = lane; e < E; e += kWave) w[e] = open[e] == -2.f ? score[e] * norm : 0.f;
+    for (int e = lane; e < E; e += kWave) w[e] = taken[e] != 0.f ? score[e] * norm : 0.f;
 }
 
 extern "C" int ts_route_experts(const float* logits, float* weights, int rows, int experts,
@@ -84,7 +92,7 @@ extern "C" int ts_route_experts(const float* logits, float* weights, int rows, i
       group_keep > group_count || top <= 0 || top > group_keep * (experts / group_count))
     TS_FAIL("route_experts: %d experts in %d groups, %d kept, cannot give %d", experts,
             group_count, group_keep, top);
-  const size_t lds = (size_t)4 * (2 * experts + group_count) * sizeof(float);
+  const size_t lds = (size_t)4 * (3 * experts + group_count) * sizeof(float);
   if (lds > 64 * 1024) TS_FAIL("route_experts: %d experts are more than the kernel holds", experts);
   hipLaunchKernelGGL(route_experts_kernel, dim3((rows + 3) / 4), dim3(256), lds, stream, logits,
                      weights, rows, experts, top, group_count, group_keep, sigmoid_scores, normalize);
