@@ -366,6 +366,50 @@ def palelix_configs(s):
     return config(ff), zono
 
 
+def zolorax_configs(s):
+    """(Zolorax, Zonopel) at the width, depth, vocabulary and number of matrix parameters of
+    the size `s`.  Zolorax: recurrent layers (channels 5/4 of the width in blocks of 256) and
+    windowed attention layers in turn, every second attention layer reading the keys and
+    values of the one before it; a dense feed-forward in the recurrent layers, routed experts
+    (8, of which a token uses 2) in the attention layers; the experts' inner size takes up
+    what is left."""
+    import math
+    from tokensprint_amd.weights.random_init import declared_tensors
+    hd, heads, kv = s["head_dim"], s["heads"], s["kv_heads"]
+    lru = s["width"] * 5 // 4
+
+    def layers(expert_ff):
+        out = []
+        for i in range(s["layers"]):
+            if i % 2 == 0:
+                out.append({"type": "rglru", "mlp": {"kind": "dense", "ff": s["ff"]},
+                            "mixer": {"width": lru, "blocks": max(1, lru // 256), "conv": 4}})
+                continue
+            mixer = {"heads": heads, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                     "mask": {"size": s["window"]},
+                     "rot": {"base": 1e6, "dims": hd // 2,
+                             "scaling": {"factor": 8.0, "original": 2048, "fast": 32.0,
+                                         "slow": 1.0}}}
+            if i % 4 == 3:
+                mixer["kv_from"] = i - 2
+            out.append({"type": "attention", "mixer": mixer,
+                        "mlp": {"kind": "moe", "expert": {"ff": expert_ff},
+                                "router": {"experts": 8, "top": 2}}})
+        return out
+
+    def config(expert_ff):
+        return {"architecture": "Zolorax", "width": s["width"], "vocab": s["vocab"],
+                "norm": {"eps": 1e-6}, "layers": layers(expert_ff)}
+
+    def count(raw):
+        return sum(math.prod(d.shape) for d in declared_tensors(raw).values())
+    zono = compare_configs(s)[0]
+    spare = count(zono) - count(config(64))
+    moe_layers = s["layers"] // 2
+    ff = 64 + max(0, round(spare / (3 * s["width"] * 8 * moe_layers) / 64)) * 64
+    return config(ff), zono
+
+
 class TimedOps:
     """Wraps a kernel provider: every call of one of its operations is bracketed by events,
     and `seconds` sums them per operation name (an eager step's kernels, one by one)."""
@@ -433,8 +477,9 @@ def zonopel_profile_step(args) -> int:
     from tokensprint_amd.engine.assemble import random_model
     from tokensprint_amd.engine.runner import ModelRunner
     size = COMPARE_SIZES[args.compare_size or "1b-layers"]
-    zono = palelix_configs(size)[0] if args.profile_palelix else compare_configs(size)[0]
-    args.profile_zonopel = args.profile_zonopel or args.profile_palelix
+    zono = palelix_configs(size)[0] if args.profile_palelix else \
+        zolorax_configs(size)[0] if args.profile_zolorax else compare_configs(size)[0]
+    args.profile_zonopel = args.profile_zonopel or args.profile_palelix or args.profile_zolorax
     _, model = random_model(zono, 0, args.dtype, "cuda:0")
     make = prefill_entries(2048) if args.profile_zonopel == "prefill" else decode_entries(8, 2048)
     lengths = make(None)
@@ -456,14 +501,16 @@ def zonopel_compare(args) -> int:
     import torch
     from tokensprint_amd.engine.assemble import random_model
     page, T, b, ctx = 16, 2048, 8, 2048
-    pair = ("palelix", "zonopel") if args.compare_palelix else ("zonopel", "qwen3")
+    pair = ("palelix", "zonopel") if args.compare_palelix else \
+        ("zolorax", "zonopel") if args.compare_zolorax else ("zonopel", "qwen3")
     out = {"metric": f"{pair[0]} beside {pair[1]} at equal sizes (random weights, bf16)",
            "sizes": {}}
     for name, size in COMPARE_SIZES.items():
         if args.compare_size and name != args.compare_size:
             continue
         row = {}
-        configs = palelix_configs(size) if args.compare_palelix else compare_configs(size)
+        configs = palelix_configs(size) if args.compare_palelix else \
+            zolorax_configs(size) if args.compare_zolorax else compare_configs(size)
         for design, raw in zip(pair, configs):
             _, model = random_model(raw, 0, args.dtype, "cuda:0")
             vocab = size["vocab"]
@@ -519,6 +566,11 @@ def main() -> int:
     ap.add_argument("--compare-palelix", action="store_true",
                     help="instead of the benchmark: Palelix beside Zonopel at equal sizes "
                          "(prefill and decode throughput, time per kind of kernel)")
+    ap.add_argument("--compare-zolorax", action="store_true",
+                    help="instead of the benchmark: Zolorax beside Zonopel at equal sizes "
+                         "(prefill and decode throughput, time per kind of kernel)")
+    ap.add_argument("--profile-zolorax", default=None, choices=["prefill", "decode"],
+                    help="as --profile-zonopel, for the Zolorax model of --compare-size")
     ap.add_argument("--profile-palelix", default=None, choices=["prefill", "decode"],
                     help="as --profile-zonopel, for the Palelix model of --compare-size")
     ap.add_argument("--compare-size", default=None, help="with --compare-...: one size only")
@@ -533,9 +585,9 @@ def main() -> int:
     import torch
     from tokensprint_amd.config import load_named_config
 
-    if args.profile_zonopel or args.profile_palelix:
+    if args.profile_zonopel or args.profile_palelix or args.profile_zolorax:
         return zonopel_profile_step(args)
-    if args.compare_zonopel or args.compare_palelix:
+    if args.compare_zonopel or args.compare_palelix or args.compare_zolorax:
         return zonopel_compare(args)
     raw = load_named_config(args.model)
     full_layers = raw["num_hidden_layers"]

@@ -318,7 +318,10 @@ class TorchOps:
     def rglru_gates(self, u, w_a, w_i, b_a, b_i, rate):
         T, width = u.shape
         blocks, bw = w_a.shape[0], w_a.shape[1]
-        ub = u.float().view(T, blocks, bw)
+        # (bfloat16 matrices in blocks of a multiple of 16 run on the matrix cores, whose
+        # operands are bfloat16: the gates' products read the input rounded; the feed does not)
+        rounded = u.to(torch.bfloat16) if w_a.dtype == torch.bfloat16 and bw % 16 == 0 else u
+        ub = rounded.float().view(T, blocks, bw)
         r = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, w_a.float()).reshape(T, width) + b_a)
         i = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, w_i.float()).reshape(T, width) + b_i)
         log_a = rate * r

@@ -92,3 +92,23 @@ def test_palelix_and_zonopel_are_compared_at_equal_size():
         assert len(pale["layers"]) == len(zono["layers"])
         assert {e["type"] for e in pale["layers"]} == {"delta", "lightning", "parallel"}
         assert {e["mlp"]["kind"] for e in pale["layers"]} == {"dense", "moe"}
+
+
+def test_zolorax_and_zonopel_are_compared_at_equal_size():
+    """`bench.py --compare-zolorax` builds a Zolorax and a Zonopel configuration per size with
+    the same width, depth, vocabulary and (within 2 %) number of parameters, both kinds of
+    mixer, a layer that reads another's keys, and both kinds of feed-forward."""
+    import math
+
+    import bench
+    from tokensprint_amd.weights.random_init import declared_tensors
+    for name, size in bench.COMPARE_SIZES.items():
+        zolo, zono = bench.zolorax_configs(size)
+        count = [sum(math.prod(d.shape) for d in declared_tensors(raw).values())
+                 for raw in (zolo, zono)]
+        assert abs(count[0] - count[1]) <= 0.02 * count[0], (name, count)
+        assert zolo["width"] == zono["width"] and zolo["vocab"] == zono["vocab"]
+        assert len(zolo["layers"]) == len(zono["layers"])
+        assert {e["type"] for e in zolo["layers"]} == {"rglru", "attention"}
+        assert any("kv_from" in e["mixer"] for e in zolo["layers"])
+        assert {e["mlp"]["kind"] for e in zolo["layers"]} == {"dense", "moe"}

@@ -107,6 +107,99 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(
   }
 }
 
+// The same on the matrix cores, for bfloat16 weights and blocks whose size is a multiple of
+// 16: D = W U^T by v_mfma_f32_16x16x32_bf16, the first operand 16 output channels of a
+// gate's matrix straight from global memory (lane (r, g), r = lane % 16, g = lane / 16, holds
+// W[channel r][k = g * 8 .. + 7]), the second 16 tokens' inputs, rounded to bfloat16 and
+// staged in LDS for all of the workgroup's waves; lane (r, g) then holds D[channel g * 4 +
+// e][token r], e = 0 .. 3: four neighbouring channels of one token, written as one 16-byte
+// store.  A workgroup takes kGateTokens tokens of one block and 16 channels a wave; K runs
+// in chunks of kGateChunk inputs (a wave's weights of a chunk stay in registers over the
+// token tiles).  The sums are float32, in the order of K whatever else is in the launch;
+// sigmoid, decay and feed are float32 on them and on the unrounded input.
+constexpr int kGateTokens = 64, kGateChunk = 256, kGateStride = kGateChunk + 8;
+
+__global__ __launch_bounds__(256) void rglru_gates_mfma_kernel(
+    const float* __restrict__ u, const bf16_t* __restrict__ wa, const bf16_t* __restrict__ wi,
+    const float* __restrict__ ba, const float* __restrict__ bi, const float* __restrict__ rate,
+    float* __restrict__ a_out, float* __restrict__ x_out, int T, int width, int bw, int tiles) {
+  __shared__ __attribute__((aligned(16))) bf16_t u_s[kGateTokens * kGateStride];
+  constexpr int NT = kGateTokens / 16, KS = kGateChunk / 32;
+  const int nwaves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int r = lane % 16, g = lane / 16;
+  const int per_block = (bw / 16 + nwaves - 1) / nwaves;       // workgroups a block
+  const int b = blockIdx.y / per_block;
+  const int ct = (blockIdx.y % per_block) * nwaves + wave;      // the wave's tile of 16 channels
+  const bool has_tile = ct * 16 < bw;
+  const int t0 = blockIdx.x * kGateTokens;
+  const int nt_used = min(NT, (min(T - t0, kGateTokens) + 15) / 16);
+  (void)tiles;
+  f32x4_lru acc[NT][2];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) acc[nt][0] = acc[nt][1] = f32x4_lru{0.f, 0.f, 0.f, 0.f};
+  const bf16x8_lru zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int64_t wrow = ((int64_t)b * bw + ct * 16 + r) * bw;    // this lane's weight row
+  for (int kc = 0; kc < bw; kc += kGateChunk) {
+    const int len = min(kGateChunk, bw - kc);
+    __syncthreads();                           // the chunk before has been read
+    for (int idx = threadIdx.x; idx < nt_used * 16 * (kGateChunk / 8); idx += blockDim.x) {
+      const int tt = idx / (kGateChunk / 8), k8 = (idx % (kGateChunk / 8)) * 8;
+      bf16x8_lru v = zero8;
+      if (t0 + tt < T && k8 < len) {
+        const float* src = u + (int64_t)(t0 + tt) * width + b * bw + kc + k8;
+        const f32x4_lru lo = *(const f32x4_lru*)src, hi = *(const f32x4_lru*)(src + 4);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { v[k] = (bf16_t)lo[k]; v[4 + k] = (bf16_t)hi[k]; }
+      }
+      *(bf16x8_lru*)(u_s + tt * kGateStride + k8) = v;
+    }
+    bf16x8_lru ra[KS], ri[KS];
+#pragma unroll
+    for (int s2 = 0; s2 < KS; ++s2) {
+      const int k = s2 * 32 + g * 8;
+      const bool ok = has_tile && k < len;
+      ra[s2] = ok ? *(const bf16x8_lru*)(wa + wrow + kc + k) : zero8;
+      ri[s2] = ok ? *(const bf16x8_lru*)(wi + wrow + kc + k) : zero8;
+    }
+    __syncthreads();
+    if (!has_tile) continue;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      if (nt < nt_used) {
+#pragma unroll
+        for (int s2 = 0; s2 < KS; ++s2) {
+          if (s2 * 32 < len) {
+            const bf16x8_lru uo =
+                *(const bf16x8_lru*)(u_s + (nt * 16 + r) * kGateStride + s2 * 32 + g * 8);
+            acc[nt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ra[s2], uo, acc[nt][0], 0, 0, 0);
+            acc[nt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ri[s2], uo, acc[nt][1], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  if (!has_tile) return;
+  const int c = b * bw + ct * 16 + g * 4;                       // four channels from here
+  const f32x4_lru rb = *(const f32x4_lru*)(ba + c), ib = *(const f32x4_lru*)(bi + c),
+                  rt = *(const f32x4_lru*)(rate + c);
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int t = t0 + nt * 16 + r;
+    if (nt >= nt_used || t >= T) continue;
+    const f32x4_lru uv = *(const f32x4_lru*)(u + (int64_t)t * width + c);
+    f32x4_lru av, xv;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float rr = sigmoid_f(acc[nt][0][e] + rb[e]), gg = sigmoid_f(acc[nt][1][e] + ib[e]);
+      const float log_a = rt[e] * rr;
+      av[e] = expf(log_a);
+      xv[e] = sqrtf(-expm1f(2.0f * log_a)) * gg * uv[e];
+    }
+    *(f32x4_lru*)(a_out + (int64_t)t * width + c) = av;
+    *(f32x4_lru*)(x_out + (int64_t)t * width + c) = xv;
+  }
+}
+
 // ---------------------------------------------------------------- recurrence
 // Walk: a thread per (entry, channel) takes the entry's tokens in order.
 template <typename T>
@@ -122,6 +215,7 @@ __global__ __launch_bounds__(256) void rglru_walk_kernel(
   float* st = state + (int64_t)b.slot_ids[e] * width + c;
   float S = b.positions[first] > 0 ? *st : 0.f;
   const float yb = ybias ? ybias[c] : 0.f;
+#pragma unroll 4
   for (int t = first; t < end; ++t) {
     S = fmaf(a[(int64_t)t * width + c], S, x[(int64_t)t * width + c]);
     out[(int64_t)t * width + c] = from_f32<T>(S * gelu_tanh_f(yproj[(int64_t)t * ld + ycol + c] + yb));
@@ -139,6 +233,7 @@ __global__ __launch_bounds__(256) void rglru_local_kernel(
   const int k = (int)(idx / width), c = (int)(idx % width);
   const int first = chunks[3 * k], end = chunks[3 * k + 1];
   float S = 0.f, P = 1.f;
+#pragma unroll 8
   for (int t = first; t < end; ++t) {
     const float at = a[(int64_t)t * width + c];
     S = fmaf(at, S, x[(int64_t)t * width + c]);
@@ -182,6 +277,7 @@ __global__ __launch_bounds__(256) void rglru_output_kernel(
   const int first = chunks[3 * k], end = chunks[3 * k + 1];
   float S = chunk_state[idx];
   const float yb = ybias ? ybias[c] : 0.f;
+#pragma unroll 8
   for (int t = first; t < end; ++t) {
     S = fmaf(a[(int64_t)t * width + c], S, x[(int64_t)t * width + c]);
     out[(int64_t)t * width + c] = from_f32<T>(S * gelu_tanh_f(yproj[(int64_t)t * ld + ycol + c] + yb));
@@ -200,6 +296,19 @@ extern "C" int ts_rglru_gates(const float* u, const void* wa, const void* wi, in
   const int bw = width / blocks;
   if (bw % 8 == 0 && ((((uintptr_t)wa | (uintptr_t)wi) & 15) != 0))
     TS_FAIL("rglru_gates: gate weights must be 16-byte aligned");
+  if (w_type == TS_BF16 && bw % 16 == 0 &&
+      ((((uintptr_t)u | (uintptr_t)ba | (uintptr_t)bi | (uintptr_t)rate | (uintptr_t)a_out |
+         (uintptr_t)x_out) & 15) == 0)) {
+    // few tokens: a wave a workgroup, so that the weights' rows are spread over the chip
+    const int waves = num_tokens <= 16 ? 1 : 4;
+    const int per_block = (bw / 16 + waves - 1) / waves;
+    const dim3 grid((num_tokens + kGateTokens - 1) / kGateTokens, blocks * per_block);
+    hipLaunchKernelGGL(rglru_gates_mfma_kernel, grid, dim3(waves * kWave), 0, stream, u,
+                       (const bf16_t*)wa, (const bf16_t*)wi, ba, bi, rate, a_out, x_out,
+                       num_tokens, width, bw, per_block);
+    TS_CHECK_LAUNCH("rglru_gates (matrix cores)");
+    return 0;
+  }
   // tokens a workgroup: as many as keep the chip busy and the inputs in LDS
   int tt = num_tokens * blocks >= 2048 ? 8 : num_tokens * blocks >= 512 ? 4 : num_tokens > 1 ? 2 : 1;
   while (tt > 1 && (size_t)tt * bw * sizeof(float) > 60 * 1024) tt /= 2;
@@ -271,9 +380,35 @@ __global__ __launch_bounds__(256) void relu_squared_kernel(const TI* __restrict_
   }
 }
 
+// Eight bfloat16 a thread: 16-byte loads and stores.
+__global__ __launch_bounds__(256) void relu_squared_bf16x8_kernel(const bf16_t* __restrict__ x,
+                                                                  bf16_t* __restrict__ out,
+                                                                  int64_t units) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < units;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const bf16x8_lru v = *(const bf16x8_lru*)(x + i * 8);
+    bf16x8_lru o;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float f = fmaxf((float)v[k], 0.f);
+      o[k] = (bf16_t)(f * f);
+    }
+    *(bf16x8_lru*)(out + i * 8) = o;
+  }
+}
+
 extern "C" int ts_relu_squared(const void* x, int x_type, void* out, int out_type, int64_t n,
                                hipStream_t stream) {
   if (n <= 0) return 0;
+  if (x_type == TS_BF16 && out_type == TS_BF16 && n % 8 == 0 &&
+      (((uintptr_t)x | (uintptr_t)out) & 15) == 0) {
+    const int64_t units = n / 8;
+    const int blocks8 = (int)((units + 255) / 256 > 16384 ? 16384 : (units + 255) / 256);
+    hipLaunchKernelGGL(relu_squared_bf16x8_kernel, dim3(blocks8), dim3(256), 0, stream,
+                       (const bf16_t*)x, (bf16_t*)out, units);
+    TS_CHECK_LAUNCH("relu_squared");
+    return 0;
+  }
   const int blocks = (int)((n + 255) / 256 > 65535 ? 65535 : (n + 255) / 256);
   TS_DISPATCH_TYPE(x_type, TI, TS_DISPATCH_TYPE(out_type, TO,
       hipLaunchKernelGGL((relu_squared_kernel<TI, TO>), dim3(blocks), dim3(256), 0, stream,

@@ -86,7 +86,7 @@ class PolyNormMLP(FeedForward):
 
 
 @register(FEED_FORWARDS, "relu2_mlp")
-class SquaredReluMLP(FeedForward):
+class SquaredReluMLP(StreamProducts, FeedForward):
     """down(relu(up(h))^2), no biases; tensors '<prefix>up' and '<prefix>down'.
 
     params: prefix, inner_dim."""
@@ -103,6 +103,18 @@ class SquaredReluMLP(FeedForward):
     def load(self, get):
         self.w_up, self.w_down = get(self.prefix + "up"), get(self.prefix + "down")
 
+    def stream_hint(self, norm):
+        return self.first_product_hint(norm, self.w_up)
+
+    def forward_from_stream(self, resid, delta, norm, batch, hint=None):
+        fused = fused_rmsnorm_of(norm)
+        if fused is None:
+            return super().forward_from_stream(resid, delta, norm, batch)
+        z, resid = self.ops.norm_linear(resid, delta, fused[0], fused[1], self.w_up,
+                                        self.ctx.dtype)
+        act = self.ops.relu_squared(z, self.ctx.dtype)
+        return self.last_product(act, self.w_down, resid, hint), resid
+
     def forward(self, h, batch):
         z = self.ops.linear(h, self.w_up, self.ctx.dtype)
         return self.ops.linear(self.ops.relu_squared(z, self.ctx.dtype), self.w_down,
@@ -110,7 +122,7 @@ class SquaredReluMLP(FeedForward):
 
 
 @register(FEED_FORWARDS, "routed_experts")
-class RoutedExperts(FeedForward):
+class RoutedExperts(StreamProducts, FeedForward):
     """`experts` small gated feed-forwards of which a token uses `top`.
 
     Router: scores = softmax over all experts of the float32 logits; experts stand in
@@ -172,7 +184,13 @@ class RoutedExperts(FeedForward):
         self.w_gate_up = torch.cat(rows, dim=0).contiguous()     # [E, gate | up] x width
         self.w_down = torch.cat(cols, dim=1).contiguous()        # width x [E, inner]
 
-    def forward(self, h, batch):
+    def forward_from_stream(self, resid, delta, norm, batch, hint=None):
+        # the router and the experts both read the normed rows: the norm is a kernel of its
+        # own; the experts' second product may add itself into the stream
+        h = norm.forward(resid) if delta is None else norm.add_forward(resid, delta)
+        return self.forward(h, batch, resid=resid, hint=hint), resid
+
+    def forward(self, h, batch, resid=None, hint=None):
         ops = self.ops
         logits = ops.linear(h, self.w_router, torch.float32)
         weights = ops.route_experts(logits, top=self.top, group_count=self.group_count,
@@ -181,4 +199,6 @@ class RoutedExperts(FeedForward):
         gate_up = ops.linear(h, self.w_gate_up, self.ctx.dtype)
         act = ops.expert_activation(gate_up, weights, self.inner, self.limit, self.ctx.dtype,
                                     weighted_input=self.gated == "silu_on_input")
+        if resid is not None and hint is not None:
+            return self.last_product(act, self.w_down, resid, hint)
         return ops.linear(act, self.w_down, torch.float32)

@@ -22,6 +22,7 @@ import math
 
 import torch
 
+from tokensprint_amd.kernels.stream import StreamProducts, fused_rmsnorm_of
 from tokensprint_amd.parts.base import (MIXERS, Mixer, SlotStateNeed, TensorDecl, build_part,
                                         flat_needs, register)
 
@@ -200,7 +201,7 @@ class GatedDeltaRule(Mixer):
 
 
 @register(MIXERS, "rglru")
-class RealGatedLRU(Mixer):
+class RealGatedLRU(StreamProducts, Mixer):
     """Two branches of `width` channels: y = gelu_tanh(W_y h + b_y), and u = a short causal
     convolution per channel (bias, no activation) of W_x h + b_x.  The channels stand in
     `blocks` equal blocks; in each, r = sigmoid(A_b u_b + a_b) and i = sigmoid(I_b u_b + i_b)
@@ -263,19 +264,35 @@ class RealGatedLRU(Mixer):
                               self.state_name + ".conv"),
                 SlotStateNeed((self.width,), torch.float32, self.state_name))
 
+    def stream_hint(self, norm):
+        return self.first_product_hint(norm, self.w_in)
+
+    def forward_from_stream(self, resid, delta, norm, batch, cache, write_cache, hint=None):
+        fused = fused_rmsnorm_of(norm)
+        if fused is None:
+            return super().forward_from_stream(resid, delta, norm, batch, cache, write_cache)
+        # the residual add and the norm inside the branches' product
+        proj, resid = self.ops.norm_linear(resid, delta, fused[0], fused[1], self.w_in,
+                                           torch.float32)
+        out = self._recur(proj, batch, cache, write_cache)
+        return self.last_product(out, self.w_o, resid, hint), resid
+
     def forward(self, h, batch, cache, write_cache):
+        out = self._recur(self.ops.linear(h, self.w_in, torch.float32), batch, cache, write_cache)
+        return self.ops.linear(out, self.w_o, torch.float32)
+
+    def _recur(self, proj, batch, cache, write_cache):
+        """proj [T, y | x] float32 -> S * gelu_tanh(y) in the activation dtype."""
         if cache is None or self.state_name not in cache.states:
             raise RuntimeError(f"{self.prefix}: the recurrence needs its per-request state")
         if not write_cache:
             raise RuntimeError(f"{self.prefix}: a recurrence cannot read another run's state")
         ops, R = self.ops, self.width
-        proj = ops.linear(h, self.w_in, torch.float32)              # [T, y | x]
         u = ops.conv_silu(proj, R, R, self.conv_w, self.conv_b, batch,
                           cache.states[self.state_name + ".conv"], in_bias=self.b_x, plain=True)
         a, fed = ops.rglru_gates(u, self.w_a, self.w_i, self.b_a, self.b_i, self.rate)
-        out = ops.rglru_scan(a, fed, proj, 0, self.b_y, batch, cache.states[self.state_name],
-                             self.ctx.dtype)
-        return ops.linear(out, self.w_o, torch.float32)
+        return ops.rglru_scan(a, fed, proj, 0, self.b_y, batch, cache.states[self.state_name],
+                              self.ctx.dtype)
 
 
 @register(MIXERS, "side_by_side")
