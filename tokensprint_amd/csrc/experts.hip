@@ -130,12 +130,50 @@ __global__ __launch_bounds__(256) void expert_activation_kernel(
   out[idx] = from_f32<T>(y);
 }
 
+// The same, eight bfloat16 a thread (inner a multiple of 8): 16-byte loads and stores.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_exp;
+__global__ __launch_bounds__(256) void expert_activation_bf16x8_kernel(
+    const bf16_t* __restrict__ gate_up, const float* __restrict__ weights,
+    bf16_t* __restrict__ out, int64_t units, int inner8, float limit, int weighted_input) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= units) return;
+  const int64_t te = idx / inner8;                // token * E + expert
+  const int i = (int)(idx % inner8) * 8;
+  const int inner = inner8 * 8;
+  const float w = weights[te];
+  bf16x8_exp y = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (w != 0.f) {
+    const bf16_t* src = gate_up + te * 2 * inner;
+    const bf16x8_exp gv = *(const bf16x8_exp*)(src + i), uv = *(const bf16x8_exp*)(src + inner + i);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (weighted_input) {
+        const float g = w * (float)gv[k], u = w * (float)uv[k];
+        y[k] = (bf16_t)(g / (1.0f + expf(-g)) * u);
+      } else {
+        const float g = fminf((float)gv[k], limit);
+        const float u = fminf(fmaxf((float)uv[k], -limit), limit);
+        y[k] = (bf16_t)(g / (1.0f + expf(-1.702f * g)) * (u + 1.0f) * w);
+      }
+    }
+  }
+  *(bf16x8_exp*)(out + idx * 8) = y;
+}
+
 extern "C" int ts_expert_activation(const void* gate_up, const float* weights, void* out, int type,
                                     int rows, int experts, int inner, float limit,
                                     int weighted_input, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (experts <= 0 || inner <= 0) TS_FAIL("expert_activation: bad sizes");
   const int64_t total = (int64_t)rows * experts * inner;
+  if (type == TS_BF16 && inner % 8 == 0 && (((uintptr_t)gate_up | (uintptr_t)out) & 15) == 0) {
+    const int64_t units = total / 8;
+    hipLaunchKernelGGL(expert_activation_bf16x8_kernel, dim3((unsigned)((units + 255) / 256)),
+                       dim3(256), 0, stream, (const bf16_t*)gate_up, weights, (bf16_t*)out, units,
+                       inner / 8, limit, weighted_input);
+    TS_CHECK_LAUNCH("expert_activation");
+    return 0;
+  }
   TS_DISPATCH_TYPE(type, T,
                    hipLaunchKernelGGL(expert_activation_kernel<T>,
                                       dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
