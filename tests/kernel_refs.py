@@ -106,7 +106,9 @@ class TorchOps:
 
     def attend(self, qkv, batch, table, cache, write_cache, *, num_heads, num_kv_heads,
                kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window,
-               defer_merge=False, sink=None):
+               defer_merge=False, sink=None, row_extra=0):
+        if row_extra:
+            qkv = qkv[:, :qkv.shape[1] - row_extra]
         q = self.qk_norm_rope_store(
             qkv, batch, table, cache if write_cache else None, num_heads=num_heads,
             num_kv_heads=kv_in_row, head_dim=head_dim, q_weight=q_weight, k_weight=k_weight,

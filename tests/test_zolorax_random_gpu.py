@@ -93,7 +93,13 @@ def test_a_drawn_configuration_runs_in_bfloat16(case, tmp_path, gpu_device):
     """The same draws in bfloat16: whole prompts and mixed steps agree with each other row by
     row (what differs between them is which kernel serves a row), and stay finite."""
     cfg, page = draw(case)
-    d = write_zolorax_model(tmp_path, cfg, case, torch.bfloat16, std=0.15, sharpen=1.0, router=8.0)
+    for layer in cfg["layers"]:
+        # every expert in use: among two dozen experts some token's best two lie within the
+        # rounding of the router's bfloat16 input, and which of the two ways of cutting meets
+        # which rounding would decide that token's row and, through its keys, later ones
+        if layer["mlp"] and layer["mlp"]["kind"] == "moe":
+            layer["mlp"]["router"]["top"] = layer["mlp"]["router"]["experts"]
+    d = write_zolorax_model(tmp_path, cfg, case, torch.bfloat16, std=0.15, sharpen=1.0)
     _, model = load_model(d, torch.bfloat16, gpu_device)
     requests = {f"r{i}": random_prompt(n, cfg["vocab"], 100 + i)
                 for i, n in enumerate([5, 17, 40, 1, 70, 131])}
@@ -110,4 +116,4 @@ def test_a_drawn_configuration_runs_in_bfloat16(case, tmp_path, gpu_device):
         scale = max(1.0, float(x.abs().max()))
         rows += x.shape[0]
         bad += int(((x - y).abs() > 0.08 * scale).any(dim=1).sum())
-    assert bad <= 0.08 * rows, f"{bad} of {rows} rows differ between the two ways of cutting"
+    assert bad <= 0.02 * rows, f"{bad} of {rows} rows differ between the two ways of cutting"

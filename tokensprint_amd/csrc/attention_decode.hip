@@ -25,7 +25,7 @@
 
 struct AttentionDecodeArgs {
   AttentionMfmaArgs m;      // tiles = null, num_tiles = entries = tokens
-  const bf16_t* qkv;        // fused: [T, (nq + 2 * kv_in_row) * hd]; else null
+  const bf16_t* qkv;        // fused: [T, (nq + 2 * kv_in_row) * hd + row_extra]; else null
   const float* q_weight;    // [hd] or null: no norm
   const float* k_weight;
   const float* cos;         // [max_pos, hd / 2] or null: no rotation
@@ -37,6 +37,7 @@ struct AttentionDecodeArgs {
   unsigned* arrivals;       // [items] zeros, or null.  Given (and the merge not deferred), the
                             // workgroup of an item that finishes last merges the splits itself
                             // and leaves the item's count at zero: no merge kernel
+  int row_extra;            // further columns of a qkv row behind the heads
 };
 
 int launch_attention_merge(const AttentionMfmaArgs& args, hipStream_t stream);
@@ -204,7 +205,7 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
   if constexpr (FUSED) {
     if (!walker) {
       prep_weight = prep_wave ? args.q_weight : args.k_weight;
-      const bf16_t* src = args.qkv + (int64_t)token * ((a.nq + 2 * args.kv_in_row) * HD) +
+      const bf16_t* src = args.qkv + (int64_t)token * ((a.nq + 2 * args.kv_in_row) * HD + args.row_extra) +
                           (int64_t)(prep_wave ? head : a.nq + kvh) * HD + g * (HD / 4);
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
@@ -267,7 +268,7 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
     // have their first key block in flight meanwhile and no registers to spare for the
     // cos, sin and norm weight slices.
     __shared__ bf16x8 s_q[KS][kWave];
-    const int row_width = (a.nq + 2 * args.kv_in_row) * HD;
+    const int row_width = (a.nq + 2 * args.kv_in_row) * HD + args.row_extra;
     const bf16_t* row = args.qkv + (int64_t)token * row_width;
     const bool rotate = args.cos != nullptr;
     if (walker) {
@@ -498,6 +499,7 @@ extern "C" int ts_attention_decode(const AttentionDecodeArgs* p, hipStream_t str
     TS_FAIL("attention_decode: splits need partial buffers");
   if (args.qkv) {
     if ((uintptr_t)args.qkv & 15) TS_FAIL("attention_decode: qkv must be 16-byte aligned");
+    if (args.row_extra < 0 || args.row_extra % 8) TS_FAIL("attention_decode: row_extra=%d must be a multiple of 8", args.row_extra);
     if ((args.cos == nullptr) != (args.sin == nullptr)) TS_FAIL("attention_decode: cos and sin go together");
     if (args.kv_in_row != 0 && args.kv_in_row != a.nkv)
       TS_FAIL("attention_decode: the row brings %d key heads, the cache has %d", args.kv_in_row, a.nkv);

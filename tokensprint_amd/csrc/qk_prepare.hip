@@ -4,7 +4,7 @@
 #include "common.h"
 
 struct QkPrepareArgs {
-  const void* qkv;       // [T, (nq + 2*nkv) * hd]
+  const void* qkv;       // [T, (nq + 2*nkv) * hd + row_extra]
   void* q_out;           // [T, nq, hd]
   void* k_dst;           // pages [num_pages, nkv, P, hd], or flat [T, nkv, hd] if !paged
   void* v_dst;           // pages [num_pages, nkv, hd, P] (transposed), or flat [T, nkv, hd]
@@ -20,6 +20,7 @@ struct QkPrepareArgs {
   int paged;             // 1: k_dst/v_dst are cache pages; 0: flat buffers
   int store_kv;          // 0: q only
   float eps;
+  int row_extra;         // further columns of a qkv row behind the heads (another product's)
 };
 
 template <typename T, typename TC>
@@ -31,7 +32,7 @@ __global__ void qk_prepare_kernel(QkPrepareArgs a) {
   const int t = (int)(item / heads);
   const int h = (int)(item % heads);
   const int hd = a.hd, half = hd / 2;
-  const int row_width = (a.nq + 2 * a.nkv) * hd;
+  const int row_width = (a.nq + 2 * a.nkv) * hd + a.row_extra;
   const int pos = a.positions[t];
 
   int src_head;       // head index inside the qkv row
@@ -121,7 +122,7 @@ __device__ __forceinline__ void v_store_tile(const QkPrepareArgs& a, int tile, i
   const int page = a.table[(int64_t)a.entry_of_token[t] * a.table_width + pos / a.page_size];
   if (page < 0) return;
   const int hd = a.hd;
-  const bf16_t* src = (const bf16_t*)a.qkv + (int64_t)t * (a.nq + 2 * a.nkv) * hd +
+  const bf16_t* src = (const bf16_t*)a.qkv + (int64_t)t * ((a.nq + 2 * a.nkv) * hd + a.row_extra) +
                       (int64_t)(a.nq + a.nkv + kvh) * hd;
   bf16_t* dst = (bf16_t*)a.v_dst + ((int64_t)page * a.nkv + kvh) * a.page_size * hd +
                 pos % a.page_size;
@@ -171,7 +172,7 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(QkPrepareArgs a, in
     const int64_t it = p.live ? item : 0;
     p.t = (int)(it / heads), p.h = (int)(it % heads);
     p.kind = p.h < a.nq ? 0 : (p.h < a.nq + a.nkv ? 1 : 2);
-    const bf16_t* src = (const bf16_t*)a.qkv + (int64_t)p.t * (a.nq + 2 * a.nkv) * hd + (int64_t)p.h * hd;
+    const bf16_t* src = (const bf16_t*)a.qkv + (int64_t)p.t * ((a.nq + 2 * a.nkv) * hd + a.row_extra) + (int64_t)p.h * hd;
     p.x = *(const bf16x8_qk*)(src + sub * 8);
     p.pos = a.positions[p.t];
     const float* w = p.kind == 0 ? a.q_weight : a.k_weight;
@@ -265,6 +266,7 @@ extern "C" int ts_qk_prepare(const QkPrepareArgs* args, int act_type, int cache_
   if (a.num_tokens <= 0) return 0;
   if (a.hd <= 0 || a.hd % 2) TS_FAIL("qk_prepare: head_dim=%d must be even", a.hd);
   if (a.nq <= 0 || a.nkv < 0) TS_FAIL("qk_prepare: heads nq=%d nkv=%d", a.nq, a.nkv);
+  if (a.row_extra < 0 || a.row_extra % 8) TS_FAIL("qk_prepare: row_extra=%d must be a multiple of 8", a.row_extra);
   if ((a.cos == nullptr) != (a.sin == nullptr)) TS_FAIL("qk_prepare: cos and sin go together");
   if (a.store_kv && (a.nkv == 0 || !a.k_dst || !a.v_dst))
     TS_FAIL("qk_prepare: store_kv without key/value heads or destination");

@@ -33,7 +33,7 @@ class QkPrepareArgs(Structure):
         ("positions", c_void_p), ("entry_of_token", c_void_p), ("table", c_void_p),
         ("table_width", c_int), ("num_tokens", c_int), ("nq", c_int), ("nkv", c_int),
         ("hd", c_int), ("page_size", c_int), ("max_pos", c_int), ("paged", c_int),
-        ("store_kv", c_int), ("eps", c_float),
+        ("store_kv", c_int), ("eps", c_float), ("row_extra", c_int),
     ]
 
 
@@ -65,6 +65,7 @@ class AttentionDecodeArgs(Structure):
         ("m", AttentionMfmaArgs), ("qkv", c_void_p), ("q_weight", c_void_p),
         ("k_weight", c_void_p), ("cos", c_void_p), ("sin", c_void_p), ("eps", c_float),
         ("kv_in_row", c_int), ("defer_merge", c_int), ("arrivals", c_void_p),
+        ("row_extra", c_int),
     ]
 
 
@@ -560,15 +561,18 @@ class HipOps:
 
     # ------------------------------------------------------------ q/k preparation
     def _qk_args(self, qkv, batch, *, num_heads, kv_in_row, head_dim, q_weight, k_weight, eps,
-                 cos_sin):
+                 cos_sin, row_extra=0):
         T = qkv.shape[0]
-        self._check("qkv", qkv, self._FLOATS, shape=(T, (num_heads + 2 * kv_in_row) * head_dim))
+        if row_extra < 0 or row_extra % 8:
+            raise ValueError(f"row_extra={row_extra} must be a multiple of 8")
+        self._check("qkv", qkv, self._FLOATS,
+                    shape=(T, (num_heads + 2 * kv_in_row) * head_dim + row_extra))
         if head_dim % 2:
             raise ValueError(f"head_dim={head_dim} must be even")
         a = QkPrepareArgs()
         a.qkv = qkv.data_ptr()
         a.num_tokens, a.nq, a.nkv, a.hd = T, num_heads, kv_in_row, head_dim
-        a.eps = eps
+        a.eps, a.row_extra = eps, row_extra
         if q_weight is not None:
             a.q_weight = self._check("q norm weight", q_weight, torch.float32,
                                      shape=(head_dim,)).data_ptr()
@@ -607,10 +611,12 @@ class HipOps:
                 f"{batch.max_ctx_len} positions")
 
     def qk_norm_rope_store(self, qkv, batch, table, cache, *, num_heads, num_kv_heads,
-                           head_dim, q_weight, k_weight, eps, cos_sin):
+                           head_dim, q_weight, k_weight, eps, cos_sin, row_extra=0):
+        """`row_extra`: further columns of a qkv row behind the heads (another product's
+        results in the same rows), a multiple of 8."""
         a = self._qk_args(qkv, batch, num_heads=num_heads, kv_in_row=num_kv_heads,
                           head_dim=head_dim, q_weight=q_weight, k_weight=k_weight, eps=eps,
-                          cos_sin=cos_sin)
+                          cos_sin=cos_sin, row_extra=row_extra)
         q = torch.empty(qkv.shape[0], num_heads, head_dim, dtype=qkv.dtype, device=self.device)
         a.q_out = q.data_ptr()
         cache_type = _TYPE_CODE[qkv.dtype]
@@ -695,7 +701,7 @@ class HipOps:
 
     def attend(self, qkv, batch, table, cache, write_cache, *, num_heads, num_kv_heads,
                kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window,
-               defer_merge=False, sink=None):
+               defer_merge=False, sink=None, row_extra=0):
         """Everything between the q/k/v projection and the output projection: per-head
         norm of q and k, rotation, the write of k and v into `cache` (if `write_cache`;
         the row then brings `kv_in_row` = `num_kv_heads` key and value heads) and attention
@@ -713,14 +719,14 @@ class HipOps:
             q = self.qk_norm_rope_store(
                 qkv, batch, table, cache if write_cache else None, num_heads=num_heads,
                 num_kv_heads=kv_in_row, head_dim=head_dim, q_weight=q_weight,
-                k_weight=k_weight, eps=eps, cos_sin=cos_sin)
+                k_weight=k_weight, eps=eps, cos_sin=cos_sin, row_extra=row_extra)
             return self.paged_attention(q, batch, table, cache, num_heads=num_heads,
                                         num_kv_heads=num_kv_heads, head_dim=head_dim,
                                         scale=scale, window=window, sink=sink)
         # the same argument checks as the preparation kernel's
         qa = self._qk_args(qkv, batch, num_heads=num_heads, kv_in_row=kv_in_row,
                            head_dim=head_dim, q_weight=q_weight, k_weight=k_weight, eps=eps,
-                           cos_sin=cos_sin)
+                           cos_sin=cos_sin, row_extra=row_extra)
         self._check_cache(cache, table, batch, num_kv_heads, head_dim)
         if T != batch.num_tokens or T != batch.num_entries:
             raise ValueError("a decode step brings one token per entry")
@@ -733,6 +739,7 @@ class HipOps:
         d = AttentionDecodeArgs()
         d.qkv, d.q_weight, d.k_weight = qa.qkv, qa.q_weight, qa.k_weight
         d.cos, d.sin, d.eps, d.kv_in_row = qa.cos, qa.sin, eps, kv_in_row
+        d.row_extra = row_extra
         pending = self._attention_decode(a, batch, num_heads // num_kv_heads, d,
                                          out if defer_merge else None, window)
         return out if pending is None else UnmergedRows(pending, out.shape)

@@ -86,7 +86,7 @@ class GroupedQueryAttention(StreamProducts, Mixer):
         o = self._attend(self.ops.linear(h, self.w_qkv, self.ctx.dtype), batch, cache, write_cache)
         return self.ops.linear(o, self.w_o, self.ctx.dtype)
 
-    def _attend(self, qkv, batch, cache, write_cache):
+    def _attend(self, qkv, batch, cache, write_cache, row_extra=0):
         if cache is None:
             raise RuntimeError("gqa_attention needs a paged key/value cache")
         if write_cache and not self.own_kv:
@@ -96,12 +96,15 @@ class GroupedQueryAttention(StreamProducts, Mixer):
         table = batch.tables[cache.group]
         tables = self.position.rotary_tables() if self.position is not None else None
         fused = self.position is None or tables is not None
+        if row_extra and not fused:
+            raise RuntimeError(f"{self.prefix}: rows with further columns need a rotation table")
         if fused:
             o = ops.attend(
                 qkv, batch, table, cache, write_cache, num_heads=self.nq,
                 num_kv_heads=self.nkv, kv_in_row=nkv_here, head_dim=self.hd,
                 q_weight=self.w_qnorm, k_weight=self.w_knorm, eps=self.eps,
                 cos_sin=tables, scale=self.scale, window=self.window, sink=self.sink,
+                **({"row_extra": row_extra} if row_extra else {}),
                 # the result goes into the output projection, a product of the same provider,
                 # which may then finish attention's last stage itself: it may come back as
                 # a handle (kernels.stream.UnmergedRows) in place of a tensor
@@ -157,7 +160,6 @@ class SoftmaxAttention(GroupedQueryAttention):
         # squares, 1 / sqrt(s / dim + eps) = sqrt(dim / head) / sqrt(s / head + eps dim / head)
         self.eps = float(p.get("qk_norm_eps", 0.0)) * self.dim / self.hd
         self.cache_window = p.get("cache_window", self.window)
-        self.w_g = None
         if self.position is not None and getattr(self.position, "head_dim", self.hd) != self.hd:
             raise ValueError(f"{self.prefix}: the position encoding is laid out for heads of "
                              f"{self.position.head_dim}, this mixer's are {self.hd}")
@@ -223,25 +225,28 @@ class SoftmaxAttention(GroupedQueryAttention):
         if self.has_sink:
             self.sink = get(pre + "sink").float().contiguous()
         if self.has_gate:
-            self.w_g = heads_of(get(pre + "g"), self.nq, self.vdim, every, every).contiguous()
-
-    def stream_hint(self, norm):
-        return None if self.has_gate else super().stream_hint(norm)
+            # the gate's rows behind q, k and v: one product gives all of them
+            w_g = heads_of(get(pre + "g"), self.nq, self.vdim, every, every)
+            self.w_qkv = torch.cat([self.w_qkv, w_g], dim=0).contiguous()
 
     def forward_from_stream(self, resid, delta, norm, batch, cache, write_cache, hint=None):
-        if not self.has_gate:
+        fused = fused_rmsnorm_of(norm)
+        if not self.has_gate or fused is None:
             return super().forward_from_stream(resid, delta, norm, batch, cache, write_cache, hint)
-        # the gate reads the normed rows as the projections do: the norm is a kernel of its own
-        h = norm.forward(resid) if delta is None else norm.add_forward(resid, delta)
-        return self.forward(h, batch, cache, write_cache, resid=resid, hint=hint), resid
+        rows, resid = self.ops.norm_linear(resid, delta, fused[0], fused[1], self.w_qkv,
+                                           self.ctx.dtype)
+        return self.last_product(self._gated(rows, batch, cache, write_cache), self.w_o, resid,
+                                 hint), resid
 
-    def forward(self, h, batch, cache, write_cache, resid=None, hint=None):
+    def forward(self, h, batch, cache, write_cache):
         if not self.has_gate:
             return super().forward(h, batch, cache, write_cache)
-        ops = self.ops
-        o = self._attend(ops.linear(h, self.w_qkv, self.ctx.dtype), batch, cache, write_cache)
-        gate = ops.linear(h, self.w_g, torch.float32)
-        gated = ops.sigmoid_gate(o, gate, 0, self.ctx.dtype)
-        if resid is not None:
-            return self.last_product(gated, self.w_o, resid, hint)
-        return ops.linear(gated, self.w_o, self.ctx.dtype)
+        rows = self.ops.linear(h, self.w_qkv, self.ctx.dtype)
+        return self.ops.linear(self._gated(rows, batch, cache, write_cache), self.w_o,
+                               self.ctx.dtype)
+
+    def _gated(self, rows, batch, cache, write_cache):
+        """rows [T, q | k | v | gate] -> the heads' outputs times the gate's sigmoid."""
+        extra = self.nq * self.hd
+        o = self._attend(rows, batch, cache, write_cache, row_extra=extra)
+        return self.ops.sigmoid_gate(o, rows, rows.shape[1] - extra, self.ctx.dtype)
