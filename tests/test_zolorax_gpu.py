@@ -484,3 +484,26 @@ def test_greedy_generation_however_the_work_is_cut(setup):
         assert all(p.num_used == 0 for p in engine.runner.manager.pools)
         if not kw:
             assert engine.runner.graphs, "decode steps were not captured"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
+def test_sizes_that_are_multiples_of_nothing(gpu_device, tmp_path, dtype):
+    """Odd head sizes, a width, blocks and inner sizes that are multiples of no tile or vector
+    width: the products fall to the multiply-add kernels, heads are padded, the recurrence's
+    gates take their scalar form."""
+    att = dict(heads=3, kv_heads=3, dim=7, vdim=5, scale=0.4, rot_dims=4, base=500.0,
+               scaling=(4.0, 32, 8.0, 1.0))
+    cfg = zolorax_config(width=34, vocab=61, eps=1e-6, layers=[
+        zolorax_attention(**att, window=11, mlp=zolorax_moe(ff=9, experts=3, top=3)),
+        zolorax_rglru(width=75, blocks=3, conv=3, mlp=zolorax_dense(27)),
+        zolorax_attention(**att, window=29, kv_from=0, mlp=None),
+        zolorax_rglru(width=7, blocks=7, conv=2, mlp=zolorax_moe(ff=5, experts=2, top=2))])
+    d = write_zolorax_model(tmp_path, cfg, 11, dtype, sharpen=2.0 if dtype == torch.float32 else 1.0)
+    pcfg, w = plain.read_model_dir(d)
+    _, model = load_model(d, dtype, gpu_device)
+    requests = {"a": random_prompt(90, 61, 1), "b": random_prompt(37, 61, 2), "c": random_prompt(1, 61, 3)}
+    ref = {rid: plain.forward(pcfg, w, t).float() for rid, t in requests.items()}
+    rtol, atol = TOL[dtype]
+    compare(drives.drive_whole(runner_for(model, 16, 12), requests), ref, rtol, atol)
+    compare(drives.drive_portions(runner_for(model, 16, 12), requests), ref, rtol, atol)
+    compare(drives.drive_mixed(runner_for(model, 16, 16), requests), ref, rtol, atol)
