@@ -122,7 +122,7 @@ constexpr int kGateTokens = 64, kGateChunk = 256, kGateStride = kGateChunk + 8;
 __global__ __launch_bounds__(256) void rglru_gates_mfma_kernel(
     const float* __restrict__ u, const bf16_t* __restrict__ wa, const bf16_t* __restrict__ wi,
     const float* __restrict__ ba, const float* __restrict__ bi, const float* __restrict__ rate,
-    float* __restrict__ a_out, float* __restrict__ x_out, int T, int width, int bw, int tiles) {
+    float* __restrict__ a_out, float* __restrict__ x_out, int T, int width, int bw) {
   __shared__ __attribute__((aligned(16))) bf16_t u_s[kGateTokens * kGateStride];
   constexpr int NT = kGateTokens / 16, KS = kGateChunk / 32;
   const int nwaves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -133,7 +133,6 @@ __global__ __launch_bounds__(256) void rglru_gates_mfma_kernel(
   const bool has_tile = ct * 16 < bw;
   const int t0 = blockIdx.x * kGateTokens;
   const int nt_used = min(NT, (min(T - t0, kGateTokens) + 15) / 16);
-  (void)tiles;
   f32x4_lru acc[NT][2];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) acc[nt][0] = acc[nt][1] = f32x4_lru{0.f, 0.f, 0.f, 0.f};
@@ -305,7 +304,7 @@ extern "C" int ts_rglru_gates(const float* u, const void* wa, const void* wi, in
     const dim3 grid((num_tokens + kGateTokens - 1) / kGateTokens, blocks * per_block);
     hipLaunchKernelGGL(rglru_gates_mfma_kernel, grid, dim3(waves * kWave), 0, stream, u,
                        (const bf16_t*)wa, (const bf16_t*)wi, ba, bi, rate, a_out, x_out,
-                       num_tokens, width, bw, per_block);
+                       num_tokens, width, bw);
     TS_CHECK_LAUNCH("rglru_gates (matrix cores)");
     return 0;
   }
