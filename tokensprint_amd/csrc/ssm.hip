@@ -53,6 +53,51 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(
   out[(int64_t)t * channels + c] = plain ? acc : silu_f(acc);
 }
 
+// The same for long steps: a thread takes kConvRun consecutive tokens of one channel, so an
+// input is read once for all the taps that meet it (kept in registers) instead of once a
+// tap.  An output's sum runs over the taps in the same order as in the kernel above.
+constexpr int kConvRun = 8, kConvMaxTaps = 8;
+__global__ __launch_bounds__(256) void conv_silu_run_kernel(
+    const float* __restrict__ proj, int ld, int col, int channels, int taps,
+    const float* __restrict__ w, const float* __restrict__ bias, const float* __restrict__ state,
+    float* __restrict__ out, BatchView b, int num_tokens, const float* __restrict__ in_bias,
+    int plain) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  const int t0 = blockIdx.y * kConvRun;
+  const float ib = in_bias ? in_bias[c] : 0.f, bc = bias ? bias[c] : 0.f;
+  float wk[kConvMaxTaps], raw[kConvRun + kConvMaxTaps - 1];
+#pragma unroll
+  for (int k = 0; k < kConvMaxTaps; ++k) wk[k] = k < taps ? w[c * taps + k] : 0.f;
+  // raw[j]: the input of flat row t0 - (taps - 1) + j (whatever entry it belongs to)
+#pragma unroll
+  for (int j = 0; j < kConvRun + kConvMaxTaps - 1; ++j) {
+    const int row = t0 - (taps - 1) + j;
+    raw[j] = (j < kConvRun + taps - 1 && row >= 0 && row < num_tokens)
+                 ? proj[(int64_t)row * ld + col + c] + ib : 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < kConvRun; ++i) {
+    const int t = t0 + i;
+    if (t >= num_tokens) break;
+    const int e = b.entry_of_token[t];
+    const int first = b.q_start[e], pos = b.positions[t];
+    const float* st = state + (int64_t)b.slot_ids[e] * (taps - 1) * channels;
+    float acc = bc;
+#pragma unroll
+    for (int k = 0; k < kConvMaxTaps; ++k) {
+      if (k >= taps) break;
+      const int back = taps - 1 - k;
+      if (pos - back < 0) continue;
+      float v;
+      if (t - back >= first) v = raw[i + k];
+      else v = st[(int64_t)(taps - 1 - (first - (t - back))) * channels + c];
+      acc = fmaf(wk[k], v, acc);
+    }
+    out[(int64_t)t * channels + c] = plain ? acc : silu_f(acc);
+  }
+}
+
 // One thread per (entry, channel): the state after the portion.  Row j takes the input at
 // position end - (taps-1) + j: from the portion, from the old state further up (read before
 // any row at or above it is written: j ascends), or zero in front of the sequence.
@@ -135,10 +180,18 @@ extern "C" int ts_conv_silu(const float* proj, int ld, int col, int channels, in
     TS_CHECK_LAUNCH("conv_silu (walk)");
     return 0;
   }
-  const int64_t n = (int64_t)num_tokens * channels;
-  hipLaunchKernelGGL(conv_silu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
-                     proj, ld, col, channels, taps, w, bias, state, out, b, num_tokens, in_bias, plain);
-  TS_CHECK_LAUNCH("conv_silu");
+  if (taps <= kConvMaxTaps && num_tokens >= 256 && (num_tokens + kConvRun - 1) / kConvRun <= 65535) {
+    hipLaunchKernelGGL(conv_silu_run_kernel,
+                       dim3((unsigned)((channels + 255) / 256), (unsigned)((num_tokens + kConvRun - 1) / kConvRun)),
+                       dim3(256), 0, stream, proj, ld, col, channels, taps, w, bias, state, out, b,
+                       num_tokens, in_bias, plain);
+    TS_CHECK_LAUNCH("conv_silu (runs)");
+  } else {
+    const int64_t n = (int64_t)num_tokens * channels;
+    hipLaunchKernelGGL(conv_silu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                       proj, ld, col, channels, taps, w, bias, state, out, b, num_tokens, in_bias, plain);
+    TS_CHECK_LAUNCH("conv_silu");
+  }
   if (taps > 1) {
     const int64_t m = (int64_t)num_entries * channels;
     hipLaunchKernelGGL(conv_state_kernel, dim3((unsigned)((m + 255) / 256)), dim3(256), 0, stream,
