@@ -9,6 +9,8 @@ without a GPU.  The product never imports this file.
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 
@@ -16,8 +18,31 @@ class TorchOps:
     name = "torch-reference"
 
     # ---------------------------------------------------------------- rows
-    def embed(self, table, token_ids):
-        return table[token_ids.long()].float()
+    def embed(self, table, token_ids, scale=1.0):
+        return table[token_ids.long()].float() * scale
+
+    def add_bias(self, x, bias):
+        x[:, :bias.shape[0]].add_(bias.float())
+
+    def finish_projection(self, rows, bias, *, q_cols, k_cols, extra, values_from_keys, q_norm,
+                          k_norm, q_count, k_count, eps, out_dtype):
+        x = rows.float().clone()
+        if bias is not None:
+            x[:, :bias.shape[0]] += bias.float()
+        q, k = x[:, :q_cols], x[:, q_cols:q_cols + k_cols]
+        rest = x[:, q_cols + k_cols:]
+        values = [k.clone()] if values_from_keys else []
+
+        def normed(v, w, count):
+            if w is None:
+                return v
+            return v * torch.rsqrt(v.pow(2).sum(-1, keepdim=True) / count + eps) * w.float()
+
+        return torch.cat([normed(q, q_norm, q_count), normed(k, k_norm, k_count)] + values
+                         + [rest], dim=1).to(out_dtype).contiguous()
+
+    def add_weighted_rows(self, out, h, weights, col, count):
+        out.add_(h.float() * weights[:, col:col + count].float().sum(-1, keepdim=True))
 
     def gather_rows(self, x, rows):
         return x[rows.long()].contiguous()
@@ -106,7 +131,7 @@ class TorchOps:
 
     def attend(self, qkv, batch, table, cache, write_cache, *, num_heads, num_kv_heads,
                kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window,
-               defer_merge=False, sink=None, row_extra=0):
+               defer_merge=False, sink=None, row_extra=0, **score_options):
         if row_extra:
             qkv = qkv[:, :qkv.shape[1] - row_extra]
         q = self.qk_norm_rope_store(
@@ -115,13 +140,17 @@ class TorchOps:
             eps=eps, cos_sin=cos_sin)
         return self.paged_attention(q, batch, table, cache, num_heads=num_heads,
                                     num_kv_heads=num_kv_heads, head_dim=head_dim,
-                                    scale=scale, window=window, sink=sink)
+                                    scale=scale, window=window, sink=sink, **score_options)
 
     # ---------------------------------------------------------------- attention
     def paged_attention(self, q, batch, table, cache, *, num_heads, num_kv_heads, head_dim,
-                        scale, window, only=None, sink=None):
+                        scale, window, only=None, sink=None, chunk=None, softcap=None,
+                        slopes=None, q_temp=None):
         """`only`: compute just these flat tokens (a test's choice; the other rows of the
-        result are left unset)."""
+        result are left unset).  `chunk`: a query sees the keys of its own stretch of that
+        many positions; `softcap`: s <- cap tanh(s / cap); `slopes` [heads]: slope x distance
+        comes off a score; `q_temp` (coef, every): the query's factor 1 + coef ln(floor((p +
+        1) / every) + 1)."""
         T = q.shape[0]
         P = cache.page_size
         group = num_heads // num_kv_heads
@@ -130,6 +159,10 @@ class TorchOps:
             b = int(batch.entry_of_token[t])
             p = int(batch.positions[t])
             lo = 0 if window is None else max(0, p - window + 1)
+            if chunk is not None:
+                lo = max(lo, p // chunk * chunk)
+            temp = 1.0 if q_temp is None else \
+                1.0 + q_temp[0] * math.log((p + 1) // q_temp[1] + 1)
             keys = torch.arange(lo, p + 1, device=q.device)
             pages = table[b, keys // P].long()
             if (pages < 0).any():
@@ -137,7 +170,11 @@ class TorchOps:
             k = cache.k_pages[pages, :, keys % P].float()       # [n, nkv, hd]
             v = cache.v_pages[pages, :, :, keys % P].float()
             for j in range(num_heads):
-                s = (k[:, j // group] @ q[t, j].float()) * scale
+                s = (k[:, j // group] @ q[t, j].float()) * (scale * temp)
+                if softcap is not None:
+                    s = softcap * torch.tanh(s / softcap)
+                if slopes is not None:
+                    s = s - slopes[j].float() * (p - keys).float()
                 if sink is None:
                     out[t, j] = torch.softmax(s, dim=0) @ v[:, j // group]
                 else:       # one more score in the denominator, with nothing to add
@@ -202,6 +239,7 @@ class TorchOps:
 
     # ---------------------------------------------------------------- stream sums
     def stream_add(self, resid, a, b, row):
+        """`row`: float32 [width], or [T, width] (a row for every token)."""
         if a is not None:
             resid.add_(a.float() + b.float() if b is not None else a.float())
         if row is not None:
@@ -284,7 +322,7 @@ class TorchOps:
 
     # ---------------------------------------------------------------- routed experts
     def route_experts(self, logits, *, top, group_count=1, group_keep=1, scores="softmax",
-                      normalize=True):
+                      normalize=True, correction=None, weight_scale=1.0):
         T, E = logits.shape
         # sigmoid scores keep the logits' order: experts are ranked by the logits themselves
         rank = logits.float()
@@ -292,6 +330,8 @@ class TorchOps:
             scores = rank = torch.softmax(logits.float(), dim=-1)
         else:
             scores = torch.sigmoid(logits.float())
+        if correction is not None:
+            rank = scores + correction.float()
         per = E // group_count
         best = rank.view(T, group_count, per).max(-1).values
         kept = torch.zeros(T, group_count, dtype=torch.bool, device=logits.device)
@@ -302,9 +342,20 @@ class TorchOps:
         out = torch.zeros_like(scores)
         out.scatter_(1, chosen, picked / (picked.sum(-1, keepdim=True) + 1e-20)
                      if normalize else picked)
-        return out
+        return out * weight_scale
 
-    def expert_activation(self, gate_up, weights, inner, limit, out_dtype, weighted_input=False):
+    def expert_activation(self, gate_up, weights, inner, limit, out_dtype, weighted_input=False,
+                          form=None, experts=None, shared_inner=0):
+        if form == "silu":
+            T, E = weights.shape[0], experts
+            gu = gate_up.float()[:, :E * 2 * inner].view(T, E, 2, inner)
+            y = gu[:, :, 0] * torch.sigmoid(gu[:, :, 0]) * gu[:, :, 1] \
+                * weights.float()[:, :E, None]
+            parts = [y.view(T, E * inner)]
+            if shared_inner:
+                sg = gate_up.float()[:, E * 2 * inner:].view(T, 2, shared_inner)
+                parts.append(sg[:, 0] * torch.sigmoid(sg[:, 0]) * sg[:, 1])
+            return torch.cat(parts, dim=1).to(out_dtype).contiguous()
         T, E = weights.shape
         gu = gate_up.float().view(T, E, 2, inner)
         if weighted_input:
@@ -347,9 +398,10 @@ class TorchOps:
     def relu_squared(self, x, out_dtype):
         return torch.relu(x.float()).pow(2).to(out_dtype)
 
-    def sigmoid_gate(self, x, gate_rows, gate_col, out_dtype):
+    def sigmoid_gate(self, x, gate_rows, gate_col, out_dtype, group=1):
         n = x.shape[1]
-        return (x.float() * torch.sigmoid(gate_rows[:, gate_col:gate_col + n].float())).to(out_dtype)
+        gate = torch.sigmoid(gate_rows[:, gate_col:gate_col + n // group].float())
+        return (x.float() * gate.repeat_interleave(group, dim=1)).to(out_dtype)
 
     # ---------------------------------------------------------------- state-space mixer
     def conv_silu(self, proj, col, channels, weight, bias, batch, state, in_bias=None,

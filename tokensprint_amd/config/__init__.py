@@ -1,6 +1,7 @@
 from tokensprint_amd.config.engine_config import Config, SamplingParams
 from tokensprint_amd.config.model_config import ConfigError, Qwen3Config, read_config_json
 from tokensprint_amd.config.palelix_config import PalelixConfig
+from tokensprint_amd.config.pinedra_config import PinedraConfig
 from tokensprint_amd.config.zolorax_config import ZoloraxConfig
 from tokensprint_amd.config.zonopel_config import ZonopelConfig
 from tokensprint_amd.config.registry import (
@@ -21,7 +22,7 @@ from tokensprint_amd.config.registry import (
 )
 
 __all__ = [
-    "Config", "SamplingParams", "ConfigError", "Qwen3Config", "ZonopelConfig", "PalelixConfig", "ZoloraxConfig", "read_config_json",
+    "Config", "SamplingParams", "ConfigError", "Qwen3Config", "ZonopelConfig", "PalelixConfig", "PinedraConfig", "ZoloraxConfig", "read_config_json",
     "all_registered_models", "all_registered_repo_ids", "architecture_names",
     "get_architecture", "get_model_family", "get_model_repo_id",
     "get_models_from_family", "load_named_config", "lookup", "models_by_family", "model_is_registered",

@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import torch
 
-from tokensprint_amd.models.spec import ModelSpec
+from tokensprint_amd.models.spec import EMBEDDING_OUTPUT, ModelSpec
 import tokensprint_amd.parts  # noqa: F401  (registers the built-in parts)
 from tokensprint_amd.parts.base import (
     BLOCKS, EMBEDDINGS, HEADS, NORMS, POSITIONS, BuildContext, TensorDecl, build_part,
@@ -94,6 +94,17 @@ class Model:
         resid = self.embedding.forward_step(
             batch, caches[len(self.order)] if len(caches) > len(self.order) else None)
         delta = None
+        # the embedding's output, if a later run adds it to the stream again (the stream
+        # itself is summed into in place)
+        embedded = resid.clone() if any(run.enter == EMBEDDING_OUTPUT for run in self.order) \
+            else None
+
+        def entering(run):
+            """What enters in front of `run`: a row [width], or rows [T, width]."""
+            if run.enter == EMBEDDING_OUTPUT:
+                return embedded
+            return self.enter_tables[run.enter[0]][run.enter[1]]
+
         for r, run in enumerate(self.order):
             owner = r if run.cache_of is None else run.cache_of
             # what reads the stream after this run: the next run's block (the final norm
@@ -103,11 +114,11 @@ class Model:
             if nxt is not None and nxt.enter is not None:
                 # a row enters in front of the next run: only a reader that can be told so
                 # may have its norm taken ahead
-                next_hint = next_hint.entering(self.enter_tables[nxt.enter[0]][nxt.enter[1]]) \
+                next_hint = next_hint.entering(entering(nxt)) \
                     if hasattr(next_hint, "entering") else None
             if run.enter is not None and not getattr(delta, "entered", False):
                 # what is still to be added, then the row of this pass
-                ops.stream_add(resid, delta, None, self.enter_tables[run.enter[0]][run.enter[1]])
+                ops.stream_add(resid, delta, None, entering(run))
                 delta = None
             resid, delta = self.blocks[run.layer].forward(
                 resid, delta, batch, caches[owner], write_cache=run.cache_of is None,

@@ -59,6 +59,11 @@ class LayerSpec:
         return f"LayerSpec({self.block!r}, " + ", ".join(f"{k}={v!r}" for k, v in self.parts.items()) + ")"
 
 
+#: `Run.enter` for "the embedding's output": what the token embedding gave for the step's
+#: tokens (the stream as it was before the first run) is added to the stream again.
+EMBEDDING_OUTPUT = "embedding output"
+
+
 @dataclass(frozen=True)
 class Run:
     """One execution of a layer.
@@ -67,12 +72,13 @@ class Run:
     uses; None means its own.  A run that uses another run's cache only reads it.
     `enter` names a row of a [rows, width] tensor, (tensor name, row), that is added to the
     residual stream right before this run (a pass of a repeated stretch of layers that
-    tells the layers which pass it is); None: nothing is added.
+    tells the layers which pass it is), or is `EMBEDDING_OUTPUT` (every token's row of the
+    embedding's output is added to the token's row of the stream); None: nothing is added.
     """
 
     layer: int
     cache_of: int | None = None
-    enter: tuple[str, int] | None = None
+    enter: tuple[str, int] | str | None = None
 
 
 @dataclass(frozen=True)
@@ -104,7 +110,7 @@ class ModelSpec:
                 if self.order[run.cache_of].cache_of is not None:
                     raise ValueError(
                         f"run {r} reads the cache of run {run.cache_of}, which owns none")
-            if run.enter is not None:
+            if run.enter is not None and run.enter != EMBEDDING_OUTPUT:
                 name, row = run.enter
                 if not 0 <= row < self.enter_tables.get(name, 0):
                     raise ValueError(f"run {r} enters with row {row} of '{name}', which has "

@@ -38,6 +38,9 @@ class GroupedQueryAttention(StreamProducts, Mixer):
             raise ValueError(f"num_heads={self.nq} is not a multiple of num_kv_heads={self.nkv}")
         self.w_qkv = self.w_o = self.w_qnorm = self.w_knorm = None
         self.sink = None             # float32 [num_heads]: a score that joins every softmax
+        #: further keywords of `ops.attend` / `ops.paged_attention` (what a score is made of
+        #: beyond scale, window and sink), given only where a mixer sets them
+        self.score_options: dict = {}
 
     # -- weights
     def tensors(self):
@@ -104,7 +107,7 @@ class GroupedQueryAttention(StreamProducts, Mixer):
                 num_kv_heads=self.nkv, kv_in_row=nkv_here, head_dim=self.hd,
                 q_weight=self.w_qnorm, k_weight=self.w_knorm, eps=self.eps,
                 cos_sin=tables, scale=self.scale, window=self.window, sink=self.sink,
-                **({"row_extra": row_extra} if row_extra else {}),
+                **({"row_extra": row_extra} if row_extra else {}), **self.score_options,
                 # the result goes into the output projection, a product of the same provider,
                 # which may then finish attention's last stage itself: it may come back as
                 # a handle (kernels.stream.UnmergedRows) in place of a tensor
@@ -119,7 +122,8 @@ class GroupedQueryAttention(StreamProducts, Mixer):
                 ops.kv_store(k, v, batch, table, cache)
             o = ops.paged_attention(q, batch, table, cache, num_heads=self.nq,
                                     num_kv_heads=self.nkv, head_dim=self.hd,
-                                    scale=self.scale, window=self.window, sink=self.sink)
+                                    scale=self.scale, window=self.window, sink=self.sink,
+                                    **self.score_options)
         return o.view(T, self.nq * self.hd)
 
 
@@ -142,15 +146,39 @@ class SoftmaxAttention(GroupedQueryAttention):
     'k', 'v', 'k.norm': the run reads the cache of another).  `cache_window`: how many keys
     the cache keeps for this run and those that read it (default: `window`).
 
+    Further options: `qk_norm` "projection" (queries, and keys, are divided by the root mean
+    square over their whole projection, all heads at once, and weighed by 'q.norm' of heads x
+    dim and 'k.norm' of kv_heads x dim values); `values` "keys" (there is no 'v': a key head
+    as projected, bias included, before its norm, is the value head too; dim = vdim, no
+    position encoding); `bias`, the projections among "q", "k", "v", "o" that add a vector
+    ('q.b', ...); `gate` "head" ('g' gives one number per head, whose sigmoid multiplies the
+    whole head); `sink` "zero" (the further term of the denominator is exp(0) with no tensor
+    behind it); `chunk` (a query sees the earlier keys of its own stretch of `chunk`
+    positions, counted from position 0); `softcap` (score <- cap tanh(score / cap), after the
+    scale); `distance_bias` p (head j of H takes 2^(-p (j + 1) / H) times the distance to the
+    key off the score); `q_temp` (coef, every): the query at position n is multiplied by
+    1 + coef ln(floor((n + 1) / every) + 1).
+
     params: prefix, heads, kv_heads, dim, vdim, scale, position (a 'rope_partial' encoding
     of this head_dim, or None), window, qk_norm, qk_norm_eps, sink, gate, own_kv,
-    cache_window."""
+    cache_window, values, bias, chunk, softcap, distance_bias, q_temp."""
 
     def __init__(self, params, ctx):
         p = dict(params)
         self.dim, self.vdim = int(p["dim"]), int(p["vdim"])
-        self.normed = bool(p.get("qk_norm", False))
+        self.normed = bool(p.get("qk_norm", False)) and p.get("qk_norm") != "projection"
+        self.projection_normed = p.get("qk_norm") == "projection"
+        self.norm_eps = float(p.get("qk_norm_eps", 0.0))
         self.has_sink, self.has_gate = bool(p.get("sink", False)), bool(p.get("gate", False))
+        self.zero_sink, self.head_gate = p.get("sink") == "zero", p.get("gate") == "head"
+        self.keys_as_values = p.get("values", "own") == "keys"
+        self.biased = tuple(p.get("bias") or ())
+        if p.get("values", "own") not in ("own", "keys") or set(self.biased) - set("qkvo"):
+            raise ValueError(f"{p['prefix']}: values={p.get('values')!r}, bias={self.biased}")
+        if self.keys_as_values and (self.dim != self.vdim or p.get("position")
+                                    or "v" in self.biased or not p.get("own_kv", True)):
+            raise ValueError(f"{p['prefix']}: keys that serve as values need dim = vdim, no "
+                             "position encoding, no 'v' and a cache of their own")
         p.update(num_heads=p["heads"], num_kv_heads=p["kv_heads"],
                  head_dim=self.padded_head(self.dim, self.vdim), qk_norm=False)
         super().__init__(p, ctx)
@@ -160,6 +188,24 @@ class SoftmaxAttention(GroupedQueryAttention):
         # squares, 1 / sqrt(s / dim + eps) = sqrt(dim / head) / sqrt(s / head + eps dim / head)
         self.eps = float(p.get("qk_norm_eps", 0.0)) * self.dim / self.hd
         self.cache_window = p.get("cache_window", self.window)
+        self.q_bias = self.o_bias = self.q_proj_norm = self.k_proj_norm = None
+        if p.get("chunk") is not None:
+            self.score_options["chunk"] = int(p["chunk"])
+        if p.get("softcap") is not None:
+            self.score_options["softcap"] = float(p["softcap"])
+        if p.get("q_temp") is not None:
+            self.score_options["q_temp"] = (float(p["q_temp"][0]), int(p["q_temp"][1]))
+        if p.get("distance_bias") is not None:
+            power = float(p["distance_bias"])
+            self.score_options["slopes"] = torch.tensor(
+                [2.0 ** (-power * (j + 1) / self.nq) for j in range(self.nq)],
+                dtype=torch.float32, device=ctx.device)
+        #: the projection's rows pass a kernel of their own before attention reads them
+        self.finished = bool(set(self.biased) & set("qkv")) or self.projection_normed \
+            or self.keys_as_values
+        #: columns behind q, k and v in a row: the gate's (a multiple of 8)
+        self.extra = 0 if not self.has_gate else \
+            (-(-self.nq // 8) * 8 if self.head_gate else self.nq * self.hd)
         if self.position is not None and getattr(self.position, "head_dim", self.hd) != self.hd:
             raise ValueError(f"{self.prefix}: the position encoding is laid out for heads of "
                              f"{self.position.head_dim}, this mixer's are {self.hd}")
@@ -174,15 +220,23 @@ class SoftmaxAttention(GroupedQueryAttention):
              pre + "o": TensorDecl((W, self.nq * self.vdim))}
         if self.own_kv:
             t[pre + "k"] = TensorDecl((self.nkv * self.dim, W))
-            t[pre + "v"] = TensorDecl((self.nkv * self.vdim, W))
-        if self.normed:
-            t[pre + "q.norm"] = TensorDecl((self.dim,), role="vector")
+            if not self.keys_as_values:
+                t[pre + "v"] = TensorDecl((self.nkv * self.vdim, W))
+        if self.normed or self.projection_normed:
+            per = self.nq if self.projection_normed else 1
+            t[pre + "q.norm"] = TensorDecl((per * self.dim,), role="vector")
             if self.own_kv:
-                t[pre + "k.norm"] = TensorDecl((self.dim,), role="vector")
-        if self.has_sink:
+                per = self.nkv if self.projection_normed else 1
+                t[pre + "k.norm"] = TensorDecl((per * self.dim,), role="vector")
+        if self.has_sink and not self.zero_sink:
             t[pre + "sink"] = TensorDecl((self.nq,), role="vector", init=(-1.0, 2.0))
         if self.has_gate:
-            t[pre + "g"] = TensorDecl((self.nq * self.vdim, W))
+            t[pre + "g"] = TensorDecl((self.nq if self.head_gate else self.nq * self.vdim, W))
+        sizes = {"q": self.nq * self.dim, "k": self.nkv * self.dim, "v": self.nkv * self.vdim,
+                 "o": W}
+        for name in self.biased:
+            if name == "o" or self.own_kv or name == "q":
+                t[pre + name + ".b"] = TensorDecl((sizes[name],), role="vector", init=(-0.5, 0.5))
         return t
 
     def cache_need(self):
@@ -191,7 +245,8 @@ class SoftmaxAttention(GroupedQueryAttention):
     def load(self, get):
         pre, hd, W = self.prefix, self.hd, self.ctx.width
         q, o = get(pre + "q"), get(pre + "o")
-        k, v = (get(pre + "k"), get(pre + "v")) if self.own_kv else (None, None)
+        k = get(pre + "k") if self.own_kv else None
+        v = get(pre + "v") if self.own_kv and not self.keys_as_values else None
         if len({t.dtype for t in (q, k, v) if t is not None}) != 1:
             raise ValueError(f"{pre}: q/k/v projection weights are stored in different dtypes")
         layout = self.position.layout(self.dim) if self.position is not None \
@@ -207,9 +262,35 @@ class SoftmaxAttention(GroupedQueryAttention):
         every = torch.arange(self.vdim, device=q.device)
         rows = [heads_of(q, self.nq, self.dim, place, src)]
         if self.own_kv:
-            rows += [heads_of(k, self.nkv, self.dim, place, src),
-                     heads_of(v, self.nkv, self.vdim, every, every)]
+            rows.append(heads_of(k, self.nkv, self.dim, place, src))
+            if v is not None:
+                rows.append(heads_of(v, self.nkv, self.vdim, every, every))
         self.w_qkv = torch.cat(rows, dim=0).contiguous()
+
+        def vector_of(t, n, size, place, src):
+            """A vector over n heads of `size` values in the heads' layout (zeros elsewhere)."""
+            out = torch.zeros(n, hd, dtype=torch.float32, device=q.device)
+            if t is not None:
+                out[:, place] = t.float().view(n, size)[:, src]
+            return out.view(n * hd)
+
+        if set(self.biased) & set("qkv"):
+            # one vector over the projection's rows as the product gives them (q, k, v if it
+            # has weights of its own; nothing for the gate's columns)
+            def bias_of(name):
+                return get(pre + name + ".b") if name in self.biased else None
+            parts = [vector_of(bias_of("q"), self.nq, self.dim, place, src)]
+            if self.own_kv:
+                parts.append(vector_of(bias_of("k"), self.nkv, self.dim, place, src))
+                if v is not None:
+                    parts.append(vector_of(bias_of("v"), self.nkv, self.vdim, every, every))
+            self.q_bias = torch.cat(parts).contiguous()
+        if "o" in self.biased:
+            self.o_bias = get(pre + "o.b").float().contiguous()
+        if self.projection_normed:
+            self.q_proj_norm = vector_of(get(pre + "q.norm"), self.nq, self.dim, place, src)
+            if self.own_kv:
+                self.k_proj_norm = vector_of(get(pre + "k.norm"), self.nkv, self.dim, place, src)
         w_o = torch.zeros(W, self.nq, hd, dtype=o.dtype, device=o.device)
         w_o[:, :, :self.vdim] = o.view(W, self.nq, self.vdim)
         self.w_o = w_o.view(W, self.nq * hd).contiguous()
@@ -223,30 +304,63 @@ class SoftmaxAttention(GroupedQueryAttention):
             self.w_qnorm = laid_out(get(pre + "q.norm"))
             self.w_knorm = laid_out(get(pre + "k.norm")) if self.own_kv else None
         if self.has_sink:
-            self.sink = get(pre + "sink").float().contiguous()
+            self.sink = torch.zeros(self.nq, dtype=torch.float32, device=q.device) \
+                if self.zero_sink else get(pre + "sink").float().contiguous()
         if self.has_gate:
             # the gate's rows behind q, k and v: one product gives all of them
-            w_g = heads_of(get(pre + "g"), self.nq, self.vdim, every, every)
+            if self.head_gate:
+                g = get(pre + "g")
+                w_g = torch.zeros(self.extra, W, dtype=g.dtype, device=g.device)
+                w_g[:self.nq] = g
+            else:
+                w_g = heads_of(get(pre + "g"), self.nq, self.vdim, every, every)
             self.w_qkv = torch.cat([self.w_qkv, w_g], dim=0).contiguous()
 
     def forward_from_stream(self, resid, delta, norm, batch, cache, write_cache, hint=None):
         fused = fused_rmsnorm_of(norm)
-        if not self.has_gate or fused is None:
-            return super().forward_from_stream(resid, delta, norm, batch, cache, write_cache, hint)
+        plain = not (self.has_gate or self.finished or self.o_bias is not None)
+        if plain or fused is None or self.o_bias is not None:
+            # (Mixer's: the norm, then `forward`, for what GroupedQueryAttention's fused
+            # form does not know)
+            if plain:
+                return super().forward_from_stream(resid, delta, norm, batch, cache,
+                                                   write_cache, hint)
+            return Mixer.forward_from_stream(self, resid, delta, norm, batch, cache, write_cache)
         rows, resid = self.ops.norm_linear(resid, delta, fused[0], fused[1], self.w_qkv,
-                                           self.ctx.dtype)
-        return self.last_product(self._gated(rows, batch, cache, write_cache), self.w_o, resid,
-                                 hint), resid
+                                           torch.float32 if self.finished else self.ctx.dtype)
+        return self.last_product(self._gated(self._finish(rows), batch, cache, write_cache),
+                                 self.w_o, resid, hint), resid
 
     def forward(self, h, batch, cache, write_cache):
-        if not self.has_gate:
+        if not (self.has_gate or self.finished or self.o_bias is not None):
             return super().forward(h, batch, cache, write_cache)
-        rows = self.ops.linear(h, self.w_qkv, self.ctx.dtype)
-        return self.ops.linear(self._gated(rows, batch, cache, write_cache), self.w_o,
-                               self.ctx.dtype)
+        rows = self.ops.linear(h, self.w_qkv, torch.float32 if self.finished else self.ctx.dtype)
+        out = self.ops.linear(self._gated(self._finish(rows), batch, cache, write_cache),
+                              self.w_o, torch.float32 if self.o_bias is not None
+                              else self.ctx.dtype)
+        if self.o_bias is not None:
+            self.ops.add_bias(out, self.o_bias)
+        return out
+
+    def _finish(self, rows):
+        """The projection's float32 sums -> the rows attention reads, in the activation
+        dtype: biases added, queries and keys normed over their whole projection, the keys
+        as projected copied to where the values stand."""
+        if not self.finished:
+            return rows
+        kv = self.nkv if self.own_kv else 0
+        return self.ops.finish_projection(
+            rows, self.q_bias, q_cols=self.nq * self.hd, k_cols=kv * self.hd,
+            extra=self.extra, values_from_keys=self.keys_as_values,
+            q_norm=self.q_proj_norm, k_norm=self.k_proj_norm, q_count=self.nq * self.dim,
+            k_count=kv * self.dim, eps=self.norm_eps, out_dtype=self.ctx.dtype)
 
     def _gated(self, rows, batch, cache, write_cache):
         """rows [T, q | k | v | gate] -> the heads' outputs times the gate's sigmoid."""
-        extra = self.nq * self.hd
-        o = self._attend(rows, batch, cache, write_cache, row_extra=extra)
-        return self.ops.sigmoid_gate(o, rows, rows.shape[1] - extra, self.ctx.dtype)
+        o = self._attend(rows, batch, cache, write_cache, row_extra=self.extra)
+        if not self.has_gate:
+            return o
+        if self.head_gate:
+            return self.ops.sigmoid_gate(o, rows, rows.shape[1] - self.extra, self.ctx.dtype,
+                                         group=self.hd)
+        return self.ops.sigmoid_gate(o, rows, rows.shape[1] - self.extra, self.ctx.dtype)

@@ -17,12 +17,14 @@ from tokensprint_amd.parts.base import (EMBEDDINGS, HEADS, OutputHead, SlotState
 
 @register(EMBEDDINGS, "embedding")
 class Embedding(TokenEmbedding):
-    """params: weight (checkpoint name), vocab_size."""
+    """params: weight (checkpoint name), vocab_size, scale (a factor on every row, applied in
+    float32 as the row is read; default 1)."""
 
     def __init__(self, params, ctx):
         super().__init__(params, ctx)
         self.name = params["weight"]
         self.vocab = int(params["vocab_size"])
+        self.scale = float(params.get("scale", 1.0))
         self.table = None
 
     def tensors(self):
@@ -32,7 +34,9 @@ class Embedding(TokenEmbedding):
         self.table = get(self.name)
 
     def forward(self, token_ids):
-        return self.ops.embed(self.table, token_ids)
+        if self.scale == 1.0:
+            return self.ops.embed(self.table, token_ids)
+        return self.ops.embed(self.table, token_ids, scale=self.scale)
 
     def step_read_tensors(self):
         return []          # a step reads the rows of its tokens, not the table

@@ -142,8 +142,18 @@ class RoutedExperts(StreamProducts, FeedForward):
     weight * h: the weight multiplies what the expert reads, not what it gives; `limit` is
     not used).
 
+    Further forms: `gated` "silu" (the expert is down(silu(gate(h)) up(h)), weighed on its
+    output); `identity` n (the router has n further outputs behind the experts', whose
+    experts have no tensors and give back what they read; scores, groups and the choice run
+    over experts and these together); `correction` (a vector '<prefix>correction' over the
+    router's outputs is added to the scores for the choice of groups and experts only: the
+    weights are the scores without it); `weight_scale` (a factor on the weights);
+    `shared_inner` (one more gated unit, '<prefix>shared.*', that every token uses with the
+    weight one: its rows and columns join the experts' two products).
+
     params: prefix, inner_dim (of one expert), experts, top, group_count, group_keep (default
-    one group), limit, scores, normalize, gated."""
+    one group), limit, scores, normalize, gated, identity, correction, weight_scale,
+    shared_inner."""
 
     def __init__(self, params, ctx):
         super().__init__(params, ctx)
@@ -154,22 +164,38 @@ class RoutedExperts(StreamProducts, FeedForward):
         self.scores, self.normalize = p.get("scores", "softmax"), bool(p.get("normalize", True))
         self.gated = p.get("gated", "clamped_swish")
         if self.scores not in ("softmax", "sigmoid") or \
-                self.gated not in ("clamped_swish", "silu_on_input"):
+                self.gated not in ("clamped_swish", "silu_on_input", "silu"):
             raise ValueError(f"{self.prefix}: scores={self.scores!r}, gated={self.gated!r}")
         self.limit = float(p.get("limit", 0.0))
-        if self.experts % self.group_count or self.group_keep > self.group_count or \
-                self.top > self.group_keep * (self.experts // self.group_count):
-            raise ValueError(f"{self.prefix}: {self.experts} experts in {self.group_count} groups, "
+        self.identity = int(p.get("identity", 0))
+        self.corrected = bool(p.get("correction", False))
+        self.weight_scale = float(p.get("weight_scale", 1.0))
+        self.shared_inner = int(p["shared_inner"]) if p.get("shared_inner") else 0
+        #: what the router chooses among: the experts and the identity experts behind them
+        self.outputs = self.experts + self.identity
+        if self.outputs % self.group_count or self.group_keep > self.group_count or \
+                self.top > self.group_keep * (self.outputs // self.group_count):
+            raise ValueError(f"{self.prefix}: {self.outputs} experts in {self.group_count} groups, "
                              f"{self.group_keep} kept, cannot give {self.top}")
-        self.w_router = self.w_gate_up = self.w_down = None
+        if (self.shared_inner or self.identity) and self.gated != "silu":
+            raise ValueError(f"{self.prefix}: a shared expert and identity experts come with "
+                             "gated='silu'")
+        self.w_router = self.w_gate_up = self.w_down = self.correction = None
 
     def tensors(self):
         W, I, pre = self.ctx.width, self.inner, self.prefix
-        t = {pre + "router": TensorDecl((self.experts, W))}
+        t = {pre + "router": TensorDecl((self.outputs, W))}
         for e in range(self.experts):
             t[f"{pre}e{e}.gate"] = TensorDecl((I, W))
             t[f"{pre}e{e}.up"] = TensorDecl((I, W))
             t[f"{pre}e{e}.down"] = TensorDecl((W, I))
+        if self.corrected:
+            t[pre + "correction"] = TensorDecl((self.outputs,), role="vector", init=(-0.05, 0.05))
+        if self.shared_inner:
+            S = self.shared_inner
+            t[pre + "shared.gate"] = TensorDecl((S, W))
+            t[pre + "shared.up"] = TensorDecl((S, W))
+            t[pre + "shared.down"] = TensorDecl((W, S))
         return t
 
     def load(self, get):
@@ -179,6 +205,11 @@ class RoutedExperts(StreamProducts, FeedForward):
         for e in range(self.experts):
             rows += [get(f"{pre}e{e}.gate"), get(f"{pre}e{e}.up")]
             cols.append(get(f"{pre}e{e}.down"))
+        if self.shared_inner:
+            rows += [get(pre + "shared.gate"), get(pre + "shared.up")]
+            cols.append(get(pre + "shared.down"))
+        if self.corrected:
+            self.correction = get(pre + "correction").float().contiguous()
         if len({r.dtype for r in rows + cols}) != 1:
             raise ValueError(f"{pre}: expert weights are stored in different dtypes")
         self.w_gate_up = torch.cat(rows, dim=0).contiguous()     # [E, gate | up] x width
@@ -193,12 +224,26 @@ class RoutedExperts(StreamProducts, FeedForward):
     def forward(self, h, batch, resid=None, hint=None):
         ops = self.ops
         logits = ops.linear(h, self.w_router, torch.float32)
+        more = {}
+        if self.corrected:
+            more["correction"] = self.correction
+        if self.weight_scale != 1.0:
+            more["weight_scale"] = self.weight_scale
         weights = ops.route_experts(logits, top=self.top, group_count=self.group_count,
                                     group_keep=self.group_keep, scores=self.scores,
-                                    normalize=self.normalize)            # [T, experts]
+                                    normalize=self.normalize, **more)    # [T, outputs]
         gate_up = ops.linear(h, self.w_gate_up, self.ctx.dtype)
-        act = ops.expert_activation(gate_up, weights, self.inner, self.limit, self.ctx.dtype,
-                                    weighted_input=self.gated == "silu_on_input")
-        if resid is not None and hint is not None:
+        if self.gated == "silu":
+            act = ops.expert_activation(gate_up, weights, self.inner, self.limit, self.ctx.dtype,
+                                        form="silu", experts=self.experts,
+                                        shared_inner=self.shared_inner)
+        else:
+            act = ops.expert_activation(gate_up, weights, self.inner, self.limit, self.ctx.dtype,
+                                        weighted_input=self.gated == "silu_on_input")
+        if resid is not None and hint is not None and not self.identity:
             return self.last_product(act, self.w_down, resid, hint)
-        return ops.linear(act, self.w_down, torch.float32)
+        out = ops.linear(act, self.w_down, torch.float32)
+        if self.identity:
+            # the identity experts' share: the token itself times the sum of their weights
+            ops.add_weighted_rows(out, h, weights, self.experts, self.identity)
+        return out

@@ -10,7 +10,8 @@ from tokensprint_amd.parts.base import NORMS, Norm, TensorDecl, register
 class RMSNorm(Norm):
     """params: dim, eps, weight (checkpoint name), one_plus (the checkpoint stores the weight
     around zero and the norm multiplies by 1 + w; the sum is made once, when the weight is
-    loaded, in float32)."""
+    loaded, in float32), scalar (the checkpoint holds one number for all coordinates; it is
+    spread over `dim` values when it is loaded, so every fused form of the norm serves it)."""
 
     def __init__(self, params, ctx):
         super().__init__(params, ctx)
@@ -18,14 +19,17 @@ class RMSNorm(Norm):
         self.eps = float(params["eps"])
         self.weight_name = params["weight"]
         self.one_plus = bool(params.get("one_plus", False))
+        self.scalar = bool(params.get("scalar", False))
         self.weight = None
 
     def tensors(self):
-        return {self.weight_name: TensorDecl((self.dim,), role="vector",
+        return {self.weight_name: TensorDecl(() if self.scalar else (self.dim,), role="vector",
                                              init=(-0.3, 0.3) if self.one_plus else None)}
 
     def load(self, get):
         self.weight = get(self.weight_name)
+        if self.scalar:
+            self.weight = self.weight.float().reshape(1).expand(self.dim).contiguous()
         if self.one_plus:
             self.weight = (self.weight.float() + 1.0).contiguous()
 
