@@ -230,9 +230,13 @@ __device__ __forceinline__ void load_query(TileState<HD>& t, const bf16_t* qrow,
 // PERM: the keys of the block are assigned to the rows of the two score products so that
 // lane (r, g) holds the scores of keys g * 8 .. g * 8 + 7 (row i of product b is key
 // (i / 4) * 8 + b * 4 + i % 4) instead of keys g * 4 .. + 3 of each 16-key half.
-template <int HD, bool LAZY = false, bool PERM = false>
+//
+// EXTRA: the products become scores by `x` (a cap, a distance bias, a query temperature:
+// attention.h) before the mask; they are then in units of log2 already.
+template <int HD, bool LAZY = false, bool PERM = false, bool EXTRA = false>
 __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>& b, int kb,
-                                            float scale_log2, bool interior, int g) {
+                                            float scale_log2, bool interior, int g,
+                                            const ScoreExtra* x = nullptr) {
   constexpr int KS = TileState<HD>::KS, DB = TileState<HD>::DB;
   f32x4 st[2];
 #pragma unroll
@@ -241,6 +245,16 @@ __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>&
 #pragma unroll
     for (int s = 0; s < KS; ++s)
       st[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.k[blk][s], t.q[s], st[blk], 0, 0, 0);
+  }
+  if (EXTRA) {
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = PERM ? kb + g * 8 + blk * 4 + i : kb + blk * 16 + g * 4 + i;
+        st[blk][i] = extra_score(*x, st[blk][i], t.pos - key) * 1.44269504088896341f;
+      }
+    scale_log2 = 1.f;
   }
   if (!interior) {
     asm volatile("" ::: "memory");   // keeps this a branch: blended in, it costs every block

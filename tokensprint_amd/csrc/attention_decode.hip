@@ -231,7 +231,7 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
     }
   }
   const int last = new_key ? pos - 1 : pos;                   // last key walked from the cache
-  const int lo = (a.window > 0) ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_visible(a, pos);
   // chunks of this split: the arithmetic of attention_merge (from pos, not from last)
   const int c_first = lo / kChunk, c_last = pos / kChunk;
   const int per = (c_last - c_first + ma.num_splits) / ma.num_splits;

@@ -36,7 +36,9 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
   const int kvh = h / (a.nq / a.nkv);
   const int hd = a.hd, P = a.page_size;
   const int pos = a.positions[t];
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_visible(a, pos);
+  const bool extras = has_score_extras(a);
+  const ScoreExtra x = score_extra(a, h, pos);
   const int* table = a.table + (int64_t)a.entry_of_token[t] * a.table_width;
   const T* q = (const T*)a.q + item * hd;
   const TC* kp = (const TC*)a.k_pages;
@@ -71,7 +73,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
         } else {
           for (int d = 0; d < hd; ++d) dot = fmaf(q_s[wave][d], to_f32(kr[d]), dot);
         }
-        s = dot * a.scale;
+        s = extras ? extra_score(x, dot, pos - j) : dot * a.scale;
       }
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -171,6 +173,8 @@ int ts_check_attention_args(const AttentionArgs& a, const char* who) {
     TS_FAIL("%s: page_size=%d table_width=%d num_pages=%d", who, a.page_size, a.table_width,
             a.num_pages);
   if (a.window < 0) TS_FAIL("%s: window=%d", who, a.window);
+  if (a.chunk < 0 || a.softcap < 0.f || a.temp_every < 0)
+    TS_FAIL("%s: chunk=%d softcap=%g temp_every=%d", who, a.chunk, a.softcap, a.temp_every);
   return 0;
 }
 

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionMfmaArg
   const int head = kvh * group + min(hh, group - 1);
   const int pos_first = uniform(a.positions[tok0]);          // positions are consecutive
   const int pos_last = pos_first + ntok - 1;
-  const int lo_all = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
+  const int lo_all = first_visible(a, pos_first);
   const float scale_log2 = a.scale * 1.44269504088896341f;
 
   TileState<HD> ts[TPW];
@@ -48,11 +48,11 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionMfmaArg
     // be the next tile's token with this tile's key range, stored over the right result)
     const bool row_ok = ti < tq && t < ntok && hh < group;
     ts[j].pos = row_ok ? pos_first + t : -1;
-    ts[j].lo = (a.window > 0) ? max(0, ts[j].pos - a.window + 1) : 0;
+    ts[j].lo = first_visible(a, ts[j].pos);
     tile_first[j] = pos_first + j * tq;
     tile_last[j] = j * tq < ntok ? pos_first + min(ntok, (j + 1) * tq) - 1 : -1;
-    tile_lo[j] = (a.window > 0) ? max(0, tile_first[j] - a.window + 1) : 0;
-    tile_lo_last[j] = (a.window > 0) ? max(0, tile_last[j] - a.window + 1) : 0;
+    tile_lo[j] = first_visible(a, tile_first[j]);
+    tile_lo_last[j] = first_visible(a, tile_last[j]);
     load_query<HD>(ts[j], (const bf16_t*)a.q +
                    ((int64_t)(tok0 + min(t, ntok - 1)) * a.nq + head) * HD, row_ok, g);
   }
@@ -136,16 +136,16 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
   const bool row_ok = r / args.rows_per_token < tq && ti < ntok && hh < group;
   const int pos_first = uniform(a.positions[tok0]);
   const int pos_last = pos_first + ntok - 1;
-  const int lo_all = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
+  const int lo_all = first_visible(a, pos_first);
   const float scale_log2 = a.scale * 1.44269504088896341f;
 
   TileState<HD> t;
   t.pos = row_ok ? pos_first + ti : -1;
-  t.lo = (a.window > 0) ? max(0, t.pos - a.window + 1) : 0;
+  t.lo = first_visible(a, t.pos);
   const int tile_first = pos_first + wave * tq;
   const int tile_last = wave * tq < ntok ? pos_first + min(ntok, (wave + 1) * tq) - 1 : -1;
-  const int tile_lo = (a.window > 0) ? max(0, tile_first - a.window + 1) : 0;
-  const int tile_lo_last = (a.window > 0) ? max(0, tile_last - a.window + 1) : 0;
+  const int tile_lo = first_visible(a, tile_first);
+  const int tile_lo_last = first_visible(a, tile_last);
   load_query<HD>(t, (const bf16_t*)a.q + ((int64_t)(tok0 + min(ti, ntok - 1)) * a.nq + head) * HD,
                  row_ok, g);
 
@@ -420,15 +420,15 @@ __global__ __launch_bounds__(256 * H, H == 1 ? 3 : 2) void attention_prefill_asy
     const bool row_ok = r / args.rows_per_token < tq && ti < ntok && hh < group;
     const int pos_first = uniform(a.positions[tok0]);
     const int pos_last = pos_first + ntok - 1;
-    const int lo_all = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
+    const int lo_all = first_visible(a, pos_first);
 
     TileState<HD> t;
     t.pos = row_ok ? pos_first + ti : -1;
-    t.lo = (a.window > 0) ? max(0, t.pos - a.window + 1) : 0;
+    t.lo = first_visible(a, t.pos);
     const int tile_first = pos_first + wave * tq;
     const int tile_last = wave * tq < ntok ? pos_first + min(ntok, (wave + 1) * tq) - 1 : -1;
-    const int tile_lo = (a.window > 0) ? max(0, tile_first - a.window + 1) : 0;
-    const int tile_lo_last = (a.window > 0) ? max(0, tile_last - a.window + 1) : 0;
+    const int tile_lo = first_visible(a, tile_first);
+    const int tile_lo_last = first_visible(a, tile_last);
     load_query<HD>(t, (const bf16_t*)a.q + ((int64_t)(tok0 + min(ti, ntok - 1)) * a.nq + head) * HD,
                    row_ok, g);
 
@@ -773,15 +773,15 @@ __device__ __forceinline__ void attention_prefill_wide(const AttentionMfmaArgs& 
     const bool row_ok = r / args.rows_per_token < tq && ti < ntok && hh < group;
     const int pos_first = pos_of[part];
     const int pos_last = pos_first + ntok - 1;
-    const int lo_all = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
+    const int lo_all = first_visible(a, pos_first);
 
     TileState<HD> t;
     t.pos = row_ok ? pos_first + ti : -1;
-    t.lo = (a.window > 0) ? max(0, t.pos - a.window + 1) : 0;
+    t.lo = first_visible(a, t.pos);
     const int tile_first = pos_first + wave * tq;
     const int tile_last = wave * tq < ntok ? pos_first + min(ntok, (wave + 1) * tq) - 1 : -1;
-    const int tile_lo = (a.window > 0) ? max(0, tile_first - a.window + 1) : 0;
-    const int tile_lo_last = (a.window > 0) ? max(0, tile_last - a.window + 1) : 0;
+    const int tile_lo = first_visible(a, tile_first);
+    const int tile_lo_last = first_visible(a, tile_last);
     if (part == 0) {
 #pragma unroll
       for (int s0 = 0; s0 < KS; ++s0) t.q[s0] = q_of[0][s0];

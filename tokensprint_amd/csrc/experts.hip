@@ -10,10 +10,13 @@
 // `sigmoid_scores`: scores = sigmoid(logits), each expert by itself, instead of the softmax;
 // groups and experts are then ranked by the logits themselves (the same order, also where
 // large logits' sigmoids round to the same number).  `normalize` 0: the weights are the
-// chosen experts' scores as they are.
+// chosen experts' scores as they are.  `correction` (float32 [E] or null): groups and experts
+// are ranked by score + correction, the weights stay the scores.  `weight_scale`: a factor on
+// the weights.
 __global__ __launch_bounds__(256) void route_experts_kernel(
     const float* __restrict__ logits, float* __restrict__ weights, int rows, int E, int top,
-    int group_count, int group_keep, int sigmoid_scores, int normalize) {
+    int group_count, int group_keep, int sigmoid_scores, int normalize,
+    const float* __restrict__ correction, float weight_scale) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int64_t t = (int64_t)blockIdx.x * (blockDim.x / kWave) + wave;
@@ -43,6 +46,8 @@ __global__ __launch_bounds__(256) void route_experts_kernel(
     const float inv = 1.0f / sum;
     for (int e = lane; e < E; e += kWave) open[e] = score[e] *= inv;
   }
+  if (correction)
+    for (int e = lane; e < E; e += kWave) open[e] = score[e] + correction[e];
   for (int e = lane; e < E; e += kWave) taken[e] = 0.f;
   __syncthreads();
   for (int g = lane; g < group_count; g += kWave) {
@@ -79,14 +84,15 @@ __global__ __launch_bounds__(256) void route_experts_kernel(
     }
     __syncthreads();
   }
-  const float norm = normalize ? 1.0f / (chosen_sum + 1e-20f) : 1.0f;
+  const float norm = (normalize ? 1.0f / (chosen_sum + 1e-20f) : 1.0f) * weight_scale;
   if (live)
     for (int e = lane; e < E; e += kWave) w[e] = taken[e] != 0.f ? score[e] * norm : 0.f;
 }
 
 extern "C" int ts_route_experts(const float* logits, float* weights, int rows, int experts,
                                 int top, int group_count, int group_keep, int sigmoid_scores,
-                                int normalize, hipStream_t stream) {
+                                int normalize, const float* correction, float weight_scale,
+                                hipStream_t stream) {
   if (rows <= 0) return 0;
   if (experts <= 0 || group_count <= 0 || experts % group_count || group_keep <= 0 ||
       group_keep > group_count || top <= 0 || top > group_keep * (experts / group_count))
@@ -94,8 +100,10 @@ extern "C" int ts_route_experts(const float* logits, float* weights, int rows, i
             group_count, group_keep, top);
   const size_t lds = (size_t)4 * (3 * experts + group_count) * sizeof(float);
   if (lds > 64 * 1024) TS_FAIL("route_experts: %d experts are more than the kernel holds", experts);
+  if (correction && sigmoid_scores) TS_FAIL("route_experts: a correction goes with softmax scores");
   hipLaunchKernelGGL(route_experts_kernel, dim3((rows + 3) / 4), dim3(256), lds, stream, logits,
-                     weights, rows, experts, top, group_count, group_keep, sigmoid_scores, normalize);
+                     weights, rows, experts, top, group_count, group_keep, sigmoid_scores, normalize,
+                     correction, weight_scale);
   TS_CHECK_LAUNCH("route_experts");
   return 0;
 }
@@ -180,5 +188,79 @@ extern "C" int ts_expert_activation(const void* gate_up, const float* weights, v
                                       (const T*)gate_up, weights, (T*)out, total, experts, inner,
                                       limit, weighted_input));
   TS_CHECK_LAUNCH("expert_activation");
+  return 0;
+}
+
+// ---------------------------------------------------------------- plain gated units
+// gate_up [rows, E x (gate | up) | shared gate | shared up] -> out [rows, E x inner | shared]:
+// silu(gate) up times the token's weight for the expert (weights [rows, ld_w], the experts'
+// in the first E columns; zeros, and no reads, where the weight is zero), and silu(gate) up
+// as it is for the `shared` columns of the unit that every token uses.
+template <typename T>
+__global__ __launch_bounds__(256) void expert_silu_kernel(
+    const T* __restrict__ gate_up, const float* __restrict__ weights, T* __restrict__ out,
+    int64_t total, int E, int inner, int shared, int ld_w) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int out_ld = E * inner + shared;
+  const int64_t t = idx / out_ld;
+  const int c = (int)(idx - t * out_ld);
+  const T* row = gate_up + t * (int64_t)(2 * out_ld);
+  float y = 0.f;
+  if (c < E * inner) {
+    const int e = c / inner, i = c - e * inner;
+    const float w = weights[t * ld_w + e];
+    if (w != 0.f) {
+      const float g = to_f32(row[e * 2 * inner + i]), u = to_f32(row[e * 2 * inner + inner + i]);
+      y = g / (1.0f + expf(-g)) * u * w;
+    }
+  } else {
+    const int i = c - E * inner;
+    const float g = to_f32(row[E * 2 * inner + i]), u = to_f32(row[E * 2 * inner + shared + i]);
+    y = g / (1.0f + expf(-g)) * u;
+  }
+  out[idx] = from_f32<T>(y);
+}
+
+extern "C" int ts_expert_silu(const void* gate_up, const float* weights, void* out, int type,
+                              int rows, int experts, int inner, int shared, int ld_w,
+                              hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (experts <= 0 || inner <= 0 || shared < 0 || ld_w < experts)
+    TS_FAIL("expert_silu: %d experts of %d, %d shared, weights of %d", experts, inner, shared, ld_w);
+  const int64_t total = (int64_t)rows * ((int64_t)experts * inner + shared);
+  TS_DISPATCH_TYPE(type, T,
+                   hipLaunchKernelGGL(expert_silu_kernel<T>, dim3((unsigned)((total + 255) / 256)),
+                                      dim3(256), 0, stream, (const T*)gate_up, weights, (T*)out,
+                                      total, experts, inner, shared, ld_w));
+  TS_CHECK_LAUNCH("expert_silu");
+  return 0;
+}
+
+// out[t] += h[t] * (weights[t][col] + ... + weights[t][col + count - 1]): the share of experts
+// that give back what they read.  out float32 [rows, width], h either type.
+template <typename T>
+__global__ __launch_bounds__(256) void add_weighted_rows_kernel(
+    float* __restrict__ out, const T* __restrict__ h, const float* __restrict__ weights,
+    int64_t total, int width, int ld_w, int col, int count) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t t = idx / width;
+  float w = 0.f;
+  for (int i = 0; i < count; ++i) w += weights[t * ld_w + col + i];
+  if (w != 0.f) out[idx] = fmaf(w, to_f32(h[idx]), out[idx]);
+}
+
+extern "C" int ts_add_weighted_rows(float* out, const void* h, int h_type, const float* weights,
+                                    int rows, int width, int ld_w, int col, int count,
+                                    hipStream_t stream) {
+  if (rows <= 0 || count <= 0) return 0;
+  if (width <= 0 || col < 0 || col + count > ld_w) TS_FAIL("add_weighted_rows: columns outside the weights");
+  const int64_t total = (int64_t)rows * width;
+  TS_DISPATCH_TYPE(h_type, T,
+                   hipLaunchKernelGGL(add_weighted_rows_kernel<T>, dim3((unsigned)((total + 255) / 256)),
+                                      dim3(256), 0, stream, out, (const T*)h, weights, total, width,
+                                      ld_w, col, count));
+  TS_CHECK_LAUNCH("add_weighted_rows");
   return 0;
 }

@@ -420,25 +420,28 @@ extern "C" int ts_relu_squared(const void* x, int x_type, void* out, int out_typ
 template <typename TX, typename TG, typename TO>
 __global__ __launch_bounds__(256) void sigmoid_gate_kernel(
     const TX* __restrict__ x, const TG* __restrict__ gate, int ld, int gate_col,
-    TO* __restrict__ out, int64_t total, int cols) {
+    TO* __restrict__ out, int64_t total, int cols, int group) {
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t r = i / cols;
-    const int c = (int)(i - r * cols);
+    const int c = (int)(i - r * cols) / group;
     out[i] = from_f32<TO>(to_f32(x[i]) * sigmoid_f(to_f32(gate[r * ld + gate_col + c])));
   }
 }
 
+// `group`: columns of x that share one gate (1: a gate a column; a head's size: a gate a head).
 extern "C" int ts_sigmoid_gate(const void* x, int x_type, const void* gate, int gate_type, int ld,
                                int gate_col, void* out, int out_type, int rows, int cols,
-                               hipStream_t stream) {
+                               int group, hipStream_t stream) {
   if (rows <= 0) return 0;
-  if (cols <= 0 || gate_col < 0 || gate_col + cols > ld) TS_FAIL("sigmoid_gate: cols=%d gate_col=%d ld=%d", cols, gate_col, ld);
+  if (cols <= 0 || group <= 0 || cols % group || gate_col < 0 || gate_col + cols / group > ld)
+    TS_FAIL("sigmoid_gate: cols=%d group=%d gate_col=%d ld=%d", cols, group, gate_col, ld);
   const int64_t total = (int64_t)rows * cols;
   const int blocks = (int)((total + 255) / 256 > 65535 ? 65535 : (total + 255) / 256);
   TS_DISPATCH_TYPE(x_type, TX, TS_DISPATCH_TYPE(gate_type, TG, TS_DISPATCH_TYPE(out_type, TO,
       hipLaunchKernelGGL((sigmoid_gate_kernel<TX, TG, TO>), dim3(blocks), dim3(256), 0, stream,
-                         (const TX*)x, (const TG*)gate, ld, gate_col, (TO*)out, total, cols))));
+                         (const TX*)x, (const TG*)gate, ld, gate_col, (TO*)out, total, cols,
+                         group))));
   TS_CHECK_LAUNCH("sigmoid_gate");
   return 0;
 }

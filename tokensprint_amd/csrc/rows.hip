@@ -5,20 +5,22 @@
 // ---------------------------------------------------------------- embedding
 template <typename TW>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
-                             float* __restrict__ out, int width) {
+                             float* __restrict__ out, int width, float scale) {
   const int64_t t = blockIdx.x;
   const TW* row = table + (int64_t)ids[t] * width;
   float* o = out + t * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = to_f32(row[i]);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = to_f32(row[i]) * scale;
 }
 
+// out[t] = table[ids[t]] * scale, in float32 (a scale of 1 changes no bit).
 extern "C" int ts_embed(const void* table, int table_type, int vocab, const int* ids,
-                        float* out, int num_tokens, int width, hipStream_t stream) {
+                        float* out, int num_tokens, int width, float scale,
+                        hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (width <= 0 || vocab <= 0) TS_FAIL("embed: bad sizes width=%d vocab=%d", width, vocab);
   TS_DISPATCH_TYPE(table_type, TW,
                    hipLaunchKernelGGL(embed_kernel<TW>, dim3(num_tokens), dim3(256), 0, stream,
-                                      (const TW*)table, ids, out, width));
+                                      (const TW*)table, ids, out, width, scale));
   TS_CHECK_LAUNCH("embed");
   return 0;
 }

@@ -2,30 +2,33 @@
 // sub-layers run side by side.
 #include "common.h"
 
-// resid += (a + b), then resid += row; a, b (either element type) and row (float32 [width])
+// resid += (a + b), then resid += row; a, b (either element type) and row (float32 [width],
+// or, `row_stride` = width, [rows, width]: a row of its own for every row of the stream)
 // may each be absent (b only with a).
 template <typename TA, typename TB>
 __global__ __launch_bounds__(256) void stream_add_kernel(
     float* __restrict__ resid, const TA* __restrict__ a, const TB* __restrict__ b,
-    const float* __restrict__ row, int64_t total, int width) {
+    const float* __restrict__ row, int row_stride, int64_t total, int width) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   float v = resid[idx];
   if (a) v += b ? to_f32(a[idx]) + to_f32(b[idx]) : to_f32(a[idx]);
-  if (row) v += row[idx % width];
+  if (row) v += row[(idx / width) * row_stride + idx % width];
   resid[idx] = v;
 }
 
 extern "C" int ts_stream_add(float* resid, const void* a, int a_type, const void* b, int b_type,
-                             const float* row, int rows, int width, hipStream_t stream) {
+                             const float* row, int row_stride, int rows, int width,
+                             hipStream_t stream) {
   if (rows <= 0) return 0;
   if (b && !a) TS_FAIL("stream_add: a second term without a first");
+  if (row_stride != 0 && row_stride != width) TS_FAIL("stream_add: row_stride=%d", row_stride);
   const int64_t total = (int64_t)rows * width;
   const dim3 grid((unsigned)((total + 255) / 256));
   TS_DISPATCH_TYPE(a ? a_type : TS_F32, TA,
     TS_DISPATCH_TYPE(b ? b_type : TS_F32, TB,
       hipLaunchKernelGGL((stream_add_kernel<TA, TB>), grid, dim3(256), 0, stream, resid,
-                         (const TA*)a, (const TB*)b, row, total, width)));
+                         (const TA*)a, (const TB*)b, row, row_stride, total, width)));
   TS_CHECK_LAUNCH("stream_add");
   return 0;
 }
@@ -36,11 +39,12 @@ extern "C" int ts_stream_add(float* resid, const void* a, int a_type, const void
 template <typename TA, typename TB, typename TO>
 __global__ __launch_bounds__(256) void stream_add_norm_kernel(
     float* __restrict__ resid, const TA* __restrict__ a, const TB* __restrict__ b,
-    const float* __restrict__ row, const float* __restrict__ w, TO* __restrict__ out, int width,
-    float eps) {
+    const float* __restrict__ row, int row_stride, const float* __restrict__ w,
+    TO* __restrict__ out, int width, float eps) {
   __shared__ float scratch[8];
   constexpr int kKeep = 8;
   const int64_t base = (int64_t)blockIdx.x * width;
+  if (row) row += (int64_t)blockIdx.x * row_stride;
   float keep[kKeep], ss = 0.f;
 #pragma unroll
   for (int j = 0; j < kKeep; ++j) {
@@ -72,18 +76,19 @@ __global__ __launch_bounds__(256) void stream_add_norm_kernel(
 }
 
 extern "C" int ts_stream_add_norm(float* resid, const void* a, int a_type, const void* b,
-                                  int b_type, const float* row, const float* w, void* out,
-                                  int out_type, int rows, int width, float eps,
+                                  int b_type, const float* row, int row_stride, const float* w,
+                                  void* out, int out_type, int rows, int width, float eps,
                                   hipStream_t stream) {
   if (rows <= 0) return 0;
+  if (row_stride != 0 && row_stride != width) TS_FAIL("stream_add_norm: row_stride=%d", row_stride);
   if (!a || !w || !out || width <= 0) TS_FAIL("stream_add_norm: a term, a weight and an output");
   const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
   TS_DISPATCH_TYPE(a_type, TA,
     TS_DISPATCH_TYPE(b ? b_type : TS_F32, TB,
       TS_DISPATCH_TYPE(out_type, TO,
         hipLaunchKernelGGL((stream_add_norm_kernel<TA, TB, TO>), dim3(rows), dim3(threads), 0,
-                           stream, resid, (const TA*)a, (const TB*)b, row, w, (TO*)out, width,
-                           eps))));
+                           stream, resid, (const TA*)a, (const TB*)b, row, row_stride, w,
+                           (TO*)out, width, eps))));
   TS_CHECK_LAUNCH("stream_add_norm");
   return 0;
 }

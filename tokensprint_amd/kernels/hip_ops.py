@@ -49,6 +49,8 @@ class AttentionArgs(Structure):
         ("table_width", c_int), ("num_tokens", c_int), ("num_entries", c_int), ("nq", c_int),
         ("nkv", c_int), ("hd", c_int), ("page_size", c_int), ("num_pages", c_int),
         ("window", c_int), ("scale", c_float), ("sink", c_void_p),
+        ("chunk", c_int), ("softcap", c_float), ("slopes", c_void_p), ("temp_coef", c_float),
+        ("temp_every", c_int),
     ]
 
 
@@ -197,13 +199,54 @@ class HipOps:
         return x.merged() if x.__class__ is UnmergedRows else x
 
     # ------------------------------------------------------------ rows
-    def embed(self, table, token_ids):
+    def embed(self, table, token_ids, scale=1.0):
+        """Rows of `table` as float32, times `scale`."""
         self._check("embedding table", table, self._FLOATS, ndim=2)
         self._check("token ids", token_ids, torch.int32, ndim=1)
         T, (V, H) = token_ids.shape[0], table.shape
         out = torch.empty(T, H, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_embed, _ptr(table), _TYPE_CODE[table.dtype], V, _ptr(token_ids),
-                   _ptr(out), T, H, self._stream())
+                   _ptr(out), T, H, c_float(scale), self._stream())
+        return out
+
+    def add_bias(self, x, bias):
+        """In place: bias (float32 [n]) is added to the first n columns of float32 rows."""
+        self._check("x", x, torch.float32, ndim=2)
+        self._check("bias", bias, torch.float32, ndim=1)
+        if bias.shape[0] > x.shape[1]:
+            raise ValueError(f"add_bias: {bias.shape[0]} biases for rows of {x.shape[1]}")
+        self._call(self.lib.ts_add_bias, _ptr(x), _ptr(bias), x.shape[0], bias.shape[0],
+                   x.shape[1], self._stream())
+
+    def finish_projection(self, rows, bias, *, q_cols, k_cols, extra, values_from_keys, q_norm,
+                          k_norm, q_count, k_count, eps, out_dtype):
+        """A q/k/v projection's float32 sums [T, q | k | v | extra] (no v with
+        `values_from_keys`) -> [T, q | k | v | extra] in `out_dtype`: `bias` (float32 over the
+        row's first columns, or None) added; q, and k, divided by the root of (their sum of
+        squares over `q_count`, `k_count`, plus eps) and weighed by `q_norm`, `k_norm`
+        (float32 [q_cols], [k_cols]; None: left as they are); with `values_from_keys` the
+        keys as they were before their norm stand where the values do."""
+        self._check("projection rows", rows, torch.float32, ndim=2)
+        T, ld = rows.shape
+        v_cols = k_cols if values_from_keys else ld - q_cols - k_cols - extra
+        if v_cols < 0 or (values_from_keys and ld != q_cols + k_cols + extra):
+            raise ValueError(f"finish_projection: rows of {ld} for q={q_cols} k={k_cols} "
+                             f"extra={extra}")
+        if bias is not None:
+            self._check("bias", bias, torch.float32, ndim=1)
+            if bias.shape[0] > ld:
+                raise ValueError("finish_projection: more biases than columns")
+        if q_norm is not None:
+            self._check("q norm weight", q_norm, torch.float32, shape=(q_cols,))
+        if k_norm is not None:
+            self._check("k norm weight", k_norm, torch.float32, shape=(k_cols,))
+        out = torch.empty(T, q_cols + k_cols + v_cols + extra, dtype=out_dtype,
+                          device=self.device)
+        self._call(self.lib.ts_finish_projection, _ptr(rows), _ptr(bias),
+                   bias.shape[0] if bias is not None else 0, _ptr(q_norm), _ptr(k_norm),
+                   _ptr(out), _TYPE_CODE[out_dtype], T, int(q_cols), int(k_cols), int(v_cols),
+                   int(extra), int(bool(values_from_keys)), int(q_count), int(k_count),
+                   c_float(eps), self._stream())
         return out
 
     def take_tokens(self, token_ids, sources, drawn):
@@ -675,9 +718,15 @@ class HipOps:
 
     # ------------------------------------------------------------ attention
     def paged_attention(self, q, batch, table, cache, *, num_heads, num_kv_heads, head_dim,
-                        scale, window, sink=None):
+                        scale, window, sink=None, chunk=None, softcap=None, slopes=None,
+                        q_temp=None):
         """`sink`: float32 [num_heads] or None: a score per query head that joins the
-        softmax's denominator once (not scaled, no key, no value)."""
+        softmax's denominator once (not scaled, no key, no value).  `chunk`: a query sees
+        the earlier keys of its own stretch of `chunk` positions, counted from position 0.
+        Scores beyond scale times the product: `softcap` c (score <- c tanh(score / c)),
+        `slopes` (float32 [num_heads]: slope times the distance to the key comes off),
+        `q_temp` (coef, every): the query at position p counts 1 + coef ln(floor((p + 1) /
+        every) + 1) times."""
         T = q.shape[0]
         self._check("q", q, self._FLOATS, shape=(T, num_heads, head_dim))
         self._check_cache(cache, table, batch, num_kv_heads, head_dim)
@@ -686,14 +735,17 @@ class HipOps:
         out = torch.empty_like(q)
         a = AttentionArgs()
         self._fill_attention_args(a, q, out, batch, table, cache, num_heads, num_kv_heads,
-                                  head_dim, scale, window, sink)
+                                  head_dim, scale, window, sink, chunk, softcap, slopes, q_temp)
+        extras = softcap is not None or slopes is not None or q_temp is not None
         if (q.dtype == torch.bfloat16 and cache.k_pages.dtype == torch.bfloat16
                 and head_dim % 16 == 0 and head_dim <= 256 and cache.page_size % 4 == 0):
-            if self._decode_fits(batch, num_kv_heads, num_heads // num_kv_heads, head_dim,
-                                 cache.page_size, False):
+            # (scores with extras are the business of one matrix-core kernel and the
+            # float32 one)
+            if not extras and self._decode_fits(batch, num_kv_heads, num_heads // num_kv_heads,
+                                                head_dim, cache.page_size, False):
                 self._attention_decode(a, batch, num_heads // num_kv_heads)
             else:
-                self._attention_mfma(a, batch, num_heads // num_kv_heads)
+                self._attention_mfma(a, batch, num_heads // num_kv_heads, extras)
         else:
             self._call(self.lib.ts_attention_generic, byref(a), _TYPE_CODE[q.dtype],
                        _TYPE_CODE[cache.k_pages.dtype], self._stream())
@@ -701,7 +753,8 @@ class HipOps:
 
     def attend(self, qkv, batch, table, cache, write_cache, *, num_heads, num_kv_heads,
                kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window,
-               defer_merge=False, sink=None, row_extra=0):
+               defer_merge=False, sink=None, row_extra=0, chunk=None, softcap=None,
+               slopes=None, q_temp=None):
         """Everything between the q/k/v projection and the output projection: per-head
         norm of q and k, rotation, the write of k and v into `cache` (if `write_cache`;
         the row then brings `kv_in_row` = `num_kv_heads` key and value heads) and attention
@@ -711,8 +764,9 @@ class HipOps:
         that shape instead of a tensor (the caller hands it to `linear_into_stream` or
         `linear`, or asks it for the tensor with `merged()`)."""
         T = qkv.shape[0]
+        extras = softcap is not None or slopes is not None or q_temp is not None
         fused = (qkv.dtype == torch.bfloat16 and cache.k_pages.dtype == torch.bfloat16
-                 and bool(write_cache) == bool(kv_in_row)
+                 and not extras and bool(write_cache) == bool(kv_in_row)
                  and self._decode_fits(batch, num_kv_heads, num_heads // num_kv_heads,
                                        head_dim, cache.page_size, True))
         if not fused:
@@ -722,7 +776,8 @@ class HipOps:
                 k_weight=k_weight, eps=eps, cos_sin=cos_sin, row_extra=row_extra)
             return self.paged_attention(q, batch, table, cache, num_heads=num_heads,
                                         num_kv_heads=num_kv_heads, head_dim=head_dim,
-                                        scale=scale, window=window, sink=sink)
+                                        scale=scale, window=window, sink=sink, chunk=chunk,
+                                        softcap=softcap, slopes=slopes, q_temp=q_temp)
         # the same argument checks as the preparation kernel's
         qa = self._qk_args(qkv, batch, num_heads=num_heads, kv_in_row=kv_in_row,
                            head_dim=head_dim, q_weight=q_weight, k_weight=k_weight, eps=eps,
@@ -733,9 +788,9 @@ class HipOps:
         out = torch.empty(T, num_heads, head_dim, dtype=qkv.dtype, device=self.device)
         a = AttentionArgs()
         self._fill_attention_args(a, None, out, batch, table, cache, num_heads, num_kv_heads,
-                                  head_dim, scale, window, sink)
-        if sink is not None:
-            defer_merge = False        # the product that merges for itself knows no sink
+                                  head_dim, scale, window, sink, chunk)
+        if sink is not None or chunk is not None:
+            defer_merge = False        # the product that merges for itself knows neither
         d = AttentionDecodeArgs()
         d.qkv, d.q_weight, d.k_weight = qa.qkv, qa.q_weight, qa.k_weight
         d.cos, d.sin, d.eps, d.kv_in_row = qa.cos, qa.sin, eps, kv_in_row
@@ -754,8 +809,9 @@ class HipOps:
         m.rows_per_token, m.head_blocks = min(group, 16), -(-group // 16)
         m.num_tiles = batch.num_entries
         items = m.num_tiles * a.nkv * m.head_blocks
-        span = batch.max_ctx_len if a.window == 0 else min(batch.max_ctx_len,
-                                                           a.window + self._attn_chunk)
+        reach = self._reach(a)
+        span = batch.max_ctx_len if reach == 0 else min(batch.max_ctx_len,
+                                                        reach + self._attn_chunk)
         m.num_splits = self._decode_splits(items, span)
         if m.num_splits > 1:
             po = torch.empty(items * m.num_splits * 16 * a.hd, dtype=torch.float32,
@@ -789,7 +845,14 @@ class HipOps:
         max_chunks = max(1, -(-span // self._attn_chunk))
         return min(max_chunks, max(1, self._units // items))
 
-    def _attention_mfma(self, a, batch, group):
+    @staticmethod
+    def _reach(a):
+        """How many keys a query sees at most (0: all earlier ones), by window and chunk."""
+        if a.window and a.chunk:
+            return min(a.window, a.chunk)
+        return a.window or a.chunk
+
+    def _attention_mfma(self, a, batch, group, extras=False):
         """Tile the batch's queries (16 rows of q heads x tokens per wavefront), choose how
         many waves share a tile's keys, and launch."""
         rows_per_token = min(group, 16)
@@ -799,7 +862,7 @@ class HipOps:
         m.base = a
         m.rows_per_token, m.head_blocks = rows_per_token, head_blocks
         # long portions of prompts: a wavefront takes several query tiles and walks alone
-        if self._prefill_tiles(batch, a.nkv, group) is not None:
+        if not extras and self._prefill_tiles(batch, a.nkv, group) is not None:
             tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
             tpw = self.lib.ts_attention_prefill_tiles(a.hd, a.page_size, tiles16,
                                                       a.nkv * head_blocks)
@@ -815,8 +878,9 @@ class HipOps:
             tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile)
         items = num_tiles * a.nkv * head_blocks
         chunk = self._attn_chunk
-        span = batch.max_ctx_len if a.window == 0 else min(batch.max_ctx_len,
-                                                           a.window + batch.max_q_len + chunk)
+        reach = self._reach(a)
+        span = batch.max_ctx_len if reach == 0 else min(batch.max_ctx_len,
+                                                        reach + batch.max_q_len + chunk)
         max_chunks = max(1, -(-span // chunk))
         # few tiles (decode): a workgroup per tile and chunk, its waves share the chunk;
         # many tiles (prompts): a wavefront per tile walks its keys
@@ -897,8 +961,24 @@ class HipOps:
         return dev
 
     def _fill_attention_args(self, a, q, out, batch, table, cache, num_heads, num_kv_heads,
-                             head_dim, scale, window, sink=None):
+                             head_dim, scale, window, sink=None, chunk=None, softcap=None,
+                             slopes=None, q_temp=None):
         T = out.shape[0]
+        if chunk is not None:
+            if int(chunk) < 1:
+                raise ValueError(f"chunk={chunk} must be positive")
+            a.chunk = int(chunk)
+        if softcap is not None:
+            if not softcap > 0:
+                raise ValueError(f"softcap={softcap} must be positive")
+            a.softcap = float(softcap)
+        if slopes is not None:
+            a.slopes = self._check("slopes", slopes, torch.float32, shape=(num_heads,)).data_ptr()
+        if q_temp is not None:
+            coef, every = q_temp
+            if int(every) < 1:
+                raise ValueError(f"q_temp: every={every} must be positive")
+            a.temp_coef, a.temp_every = float(coef), int(every)
         if sink is not None:
             a.sink = self._check("sink", sink, torch.float32, shape=(num_heads,)).data_ptr()
         a.q, a.out = (q.data_ptr() if q is not None else None), out.data_ptr()
@@ -1207,32 +1287,55 @@ class HipOps:
 
     # ------------------------------------------------------------ routed experts
     def route_experts(self, logits, *, top, group_count=1, group_keep=1, scores="softmax",
-                      normalize=True):
+                      normalize=True, correction=None, weight_scale=1.0):
         """Router logits (float32 [T, experts]) -> float32 [T, experts]: a token's weight for
         each of its `top` experts (softmax score over the chosen scores' sum), zero elsewhere.
         Only experts of the `group_keep` best of `group_count` groups of neighbours can be
         chosen (a group's score: its best expert's).  `scores` "sigmoid": an expert's score is
         the sigmoid of its logit; `normalize` False: the weights are the chosen scores as
-        they are."""
+        they are.  `correction` (float32 [experts]): groups and experts are ranked by score +
+        correction (softmax scores), the weights stay the scores; `weight_scale`: a factor on
+        the weights."""
         if scores not in ("softmax", "sigmoid"):
             raise ValueError(f"route_experts: scores={scores!r}")
         self._check("router logits", logits, torch.float32, ndim=2)
         T, E = logits.shape
+        if correction is not None:
+            self._check("correction", correction, torch.float32, shape=(E,))
         weights = torch.empty(T, E, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_route_experts, _ptr(logits), _ptr(weights), T, E, int(top),
                    int(group_count), int(group_keep), int(scores == "sigmoid"),
-                   int(bool(normalize)), self._stream())
+                   int(bool(normalize)), _ptr(correction), c_float(weight_scale), self._stream())
         return weights
 
-    def expert_activation(self, gate_up, weights, inner, limit, out_dtype, weighted_input=False):
+    def expert_activation(self, gate_up, weights, inner, limit, out_dtype, weighted_input=False,
+                          form=None, experts=None, shared_inner=0):
         """gate_up [T, experts x (gate | up)] -> [T, experts x inner]: with g = min(gate,
         limit), u = clamp(up, -limit, limit): g sigmoid(1.702 g) (u + 1) times the token's
         weight for the expert (zeros where it is zero).  `weighted_input`: the expert is a
-        plain gated unit that read the token times its weight w: silu(w gate) (w up)."""
+        plain gated unit that read the token times its weight w: silu(w gate) (w up).
+        `form` "silu": silu(gate) up times the weight; the weights' first `experts` columns
+        are the experts' (further columns belong to experts without weights), and behind the
+        experts' columns gate_up holds `shared_inner` gate and as many up columns of a unit
+        that every token uses with the weight one -> [T, experts x inner + shared_inner]."""
         gate_up = self._rows(gate_up)
         self._check("gate_up", gate_up, self._FLOATS, ndim=2)
         T = gate_up.shape[0]
         self._check("expert weights", weights, torch.float32, ndim=2)
+        if form == "silu":
+            E = weights.shape[1] if experts is None else int(experts)
+            width = E * inner + int(shared_inner)
+            if weights.shape[0] != T or E > weights.shape[1] or gate_up.shape[1] != 2 * width \
+                    or out_dtype != gate_up.dtype:
+                raise ValueError(f"expert_activation: gate_up {tuple(gate_up.shape)} for {E} "
+                                 f"experts of {inner} and {shared_inner} shared columns")
+            out = torch.empty(T, width, dtype=out_dtype, device=self.device)
+            self._call(self.lib.ts_expert_silu, _ptr(gate_up), _ptr(weights), _ptr(out),
+                       _TYPE_CODE[out_dtype], T, E, int(inner), int(shared_inner),
+                       weights.shape[1], self._stream())
+            return out
+        if form is not None:
+            raise ValueError(f"expert_activation: form={form!r}")
         E = weights.shape[1]
         if weights.shape[0] != T or gate_up.shape[1] != E * 2 * inner or out_dtype != gate_up.dtype:
             raise ValueError(f"expert_activation: gate_up {tuple(gate_up.shape)} for {E} experts "
@@ -1301,24 +1404,39 @@ class HipOps:
                    _TYPE_CODE[out_dtype], c_int64(x.numel()), self._stream())
         return out
 
-    def sigmoid_gate(self, x, gate_rows, gate_col, out_dtype):
-        """x [T, n] times the sigmoid of columns [gate_col, gate_col + n) of `gate_rows`."""
+    def sigmoid_gate(self, x, gate_rows, gate_col, out_dtype, group=1):
+        """x [T, n] times the sigmoid of columns [gate_col, gate_col + n / group) of
+        `gate_rows`: every `group` neighbouring columns of x share a gate."""
         x = self._rows(x)
         self._check("x", x, self._FLOATS, ndim=2)
         self._check("gate", gate_rows, self._FLOATS, ndim=2)
         T, n = x.shape
-        if gate_rows.shape[0] != T or gate_col < 0 or gate_col + n > gate_rows.shape[1]:
+        if group < 1 or n % group or gate_rows.shape[0] != T or gate_col < 0 \
+                or gate_col + n // group > gate_rows.shape[1]:
             raise ValueError("sigmoid_gate: gate columns outside their rows")
         out = torch.empty(T, n, dtype=out_dtype, device=self.device)
         self._call(self.lib.ts_sigmoid_gate, _ptr(x), _TYPE_CODE[x.dtype], _ptr(gate_rows),
                    _TYPE_CODE[gate_rows.dtype], gate_rows.shape[1], int(gate_col), _ptr(out),
-                   _TYPE_CODE[out_dtype], T, n, self._stream())
+                   _TYPE_CODE[out_dtype], T, n, int(group), self._stream())
         return out
+
+    def add_weighted_rows(self, out, h, weights, col, count):
+        """In place on float32 `out` [T, width]: out[t] += h[t] times the sum of columns
+        [col, col + count) of `weights` [T, n]."""
+        self._check("out", out, torch.float32, ndim=2)
+        h = self._rows(h)
+        self._check("h", h, self._FLOATS, shape=out.shape)
+        self._check("weights", weights, torch.float32, ndim=2)
+        if weights.shape[0] != out.shape[0] or col < 0 or col + count > weights.shape[1]:
+            raise ValueError("add_weighted_rows: columns outside the weights")
+        self._call(self.lib.ts_add_weighted_rows, _ptr(out), _ptr(h), _TYPE_CODE[h.dtype],
+                   _ptr(weights), out.shape[0], out.shape[1], weights.shape[1], int(col),
+                   int(count), self._stream())
 
     # ------------------------------------------------------------ sums around the stream
     def stream_add(self, resid, a, b, row):
         """In place on the float32 stream: resid += (a + b), then resid += row (float32
-        [width]); each may be None (b only with a)."""
+        [width], or [T, width]: a row for every token); each may be None (b only with a)."""
         self._check("resid", resid, torch.float32, ndim=2)
         codes = []
         for name, t in (("a", a), ("b", b)):
@@ -1327,12 +1445,20 @@ class HipOps:
                 self._check(name, t, self._FLOATS, shape=resid.shape)
             codes.append(t)
         a, b = codes
-        if row is not None:
-            self._check("row", row, torch.float32, shape=(resid.shape[1],))
         self._call(self.lib.ts_stream_add, _ptr(resid), _ptr(a),
                    _TYPE_CODE[a.dtype] if a is not None else 0, _ptr(b),
-                   _TYPE_CODE[b.dtype] if b is not None else 0, _ptr(row), resid.shape[0],
-                   resid.shape[1], self._stream())
+                   _TYPE_CODE[b.dtype] if b is not None else 0, _ptr(row),
+                   self._row_stride(row, resid), resid.shape[0], resid.shape[1], self._stream())
+
+    def _row_stride(self, row, resid):
+        """0 for a row that every row of the stream gets, the width for rows of their own."""
+        if row is None:
+            return 0
+        if row.dim() == 2:
+            self._check("rows", row, torch.float32, shape=resid.shape)
+            return resid.shape[1]
+        self._check("row", row, torch.float32, shape=(resid.shape[1],))
+        return 0
 
     def stream_add_norm(self, resid, a, b, row, norm_w, eps, out_dtype):
         """`stream_add(resid, a, b, row)` (b and row may be None), and the RMS norm (norm_w,
@@ -1343,12 +1469,12 @@ class HipOps:
         if b is not None:
             b = self._rows(b)
             self._check("b", b, self._FLOATS, shape=resid.shape)
-        if row is not None:
-            self._check("row", row, torch.float32, shape=(resid.shape[1],))
+        stride = self._row_stride(row, resid)
         self._check("norm weight", norm_w, torch.float32, shape=(resid.shape[1],))
         out = torch.empty(resid.shape, dtype=out_dtype, device=self.device)
         self._call(self.lib.ts_stream_add_norm, _ptr(resid), _ptr(a), _TYPE_CODE[a.dtype], _ptr(b),
-                   _TYPE_CODE[b.dtype] if b is not None else 0, _ptr(row), _ptr(norm_w), _ptr(out),
+                   _TYPE_CODE[b.dtype] if b is not None else 0, _ptr(row), stride, _ptr(norm_w),
+                   _ptr(out),
                    _TYPE_CODE[out_dtype], resid.shape[0], resid.shape[1], c_float(eps),
                    self._stream())
         return out
