@@ -361,3 +361,110 @@ def write_zolorax_model(folder, cfg, seed, dtype, std=0.2, sharpen=3.0, router=4
             tensors[name] = (tensors[name].float() * factor).to(tensors[name].dtype)
     save_file(tensors, str(file))
     return d
+
+
+# ------------------------------------------------------------------ Pinedra
+
+
+def pinedra_plain_attention(*, heads, kv_heads, dim, scale, mlp=None):
+    """'attention': the key projection is the value too."""
+    return {"type": "attention", "mlp": mlp,
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": scale}}
+
+
+def pinedra_distance_attention(*, heads, kv_heads, dim, vdim, scale, coef, every, mlp=None):
+    """'attention_2': distance bias, query temperature, one more term in the denominator."""
+    return {"type": "attention_2", "mlp": mlp,
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                      "scale": scale, "q_temp": {"coef": coef, "every": every}}}
+
+
+def pinedra_chunked_attention(*, heads, kv_heads, dim, vdim, scale, rot_dims, base, softcap, chunk,
+                              mlp=None):
+    """'attention_3': rotated in part, capped scores, chunks, a gate per head."""
+    return {"type": "attention_3", "mlp": mlp,
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                      "scale": scale, "rot": {"base": base, "dims": rot_dims},
+                      "softcap": softcap, "mask": {"size": chunk}}}
+
+
+def pinedra_moe(*, ff, experts, identity, top, groups, keep, scale, shared):
+    mlp = {"kind": "moe", "expert": {"ff": ff},
+           "router": {"experts": experts, "identity": identity, "top": top, "scale": scale,
+                      "groups": {"count": groups, "keep": keep}}}
+    if shared is not None:
+        mlp["shared"] = {"ff": shared}
+    return mlp
+
+
+def pinedra_config(*, width, vocab, eps, embed_scale, layers, loop=None):
+    cfg = {"architecture": "Pinedra", "width": width, "vocab": vocab, "norm": {"eps": eps},
+           "embedding": {"scale": embed_scale}, "layers": layers}
+    if loop is not None:
+        cfg["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return cfg
+
+
+# Three small models that differ in every size and option: each kind of attention first, in
+# the middle, last and inside a loop; loops over the first layers, over the last, over a
+# single layer three times, and no loop; value sizes above, below and equal to the key size;
+# one key/value head, several, and as many as query heads; chunks of 1 token, of less than
+# a page and of several pages; heads rotated in part and whole; temperatures that step every
+# token, every few tokens and never within a test's prompts; routers with and without
+# identity experts, one group and several, all groups kept and one, a shared expert of
+# another size than the experts', of the same and none; one expert a token, several, and
+# every one; layers without a feed-forward; embedding scales of 1 and others.
+_PA_MOE = dict(ff=12, experts=5, identity=1, top=2, groups=3, keep=2, scale=1.5, shared=20)
+PINE_A = pinedra_config(
+    width=40, vocab=97, eps=1e-5, embed_scale=3.0, loop=(1, 3, 2), layers=[
+        pinedra_chunked_attention(heads=4, kv_heads=2, dim=12, vdim=20, scale=0.4, rot_dims=8,
+                                  base=10000.0, softcap=5.0, chunk=7, mlp=pinedra_moe(**_PA_MOE)),
+        pinedra_plain_attention(heads=4, kv_heads=2, dim=12, scale=0.3, mlp=None),
+        pinedra_distance_attention(heads=3, kv_heads=1, dim=16, vdim=8, scale=0.25, coef=0.5,
+                                   every=4, mlp=pinedra_moe(**dict(_PA_MOE, shared=None))),
+        pinedra_chunked_attention(heads=2, kv_heads=2, dim=8, vdim=8, scale=0.5, rot_dims=8,
+                                  base=50.0, softcap=2.0, chunk=40, mlp=None),
+    ])
+PINE_B = pinedra_config(
+    width=72, vocab=131, eps=3e-6, embed_scale=1.0, loop=(0, 1, 3), layers=[
+        pinedra_distance_attention(heads=6, kv_heads=2, dim=24, vdim=24, scale=0.2, coef=0.2,
+                                   every=1, mlp=pinedra_moe(ff=16, experts=8, identity=0, top=1,
+                                                            groups=1, keep=1, scale=1.0, shared=16)),
+        pinedra_plain_attention(heads=2, kv_heads=1, dim=32, scale=0.18,
+                                mlp=pinedra_moe(ff=20, experts=3, identity=3, top=3, groups=2,
+                                                keep=2, scale=0.7, shared=8)),
+        pinedra_chunked_attention(heads=3, kv_heads=3, dim=16, vdim=24, scale=0.3, rot_dims=6,
+                                  base=300.0, softcap=30.0, chunk=1, mlp=None),
+    ])
+PINE_C = pinedra_config(
+    width=32, vocab=64, eps=1e-4, embed_scale=0.5, layers=[
+        pinedra_plain_attention(heads=1, kv_heads=1, dim=8, scale=0.5,
+                                mlp=pinedra_moe(ff=8, experts=2, identity=2, top=4, groups=4,
+                                                keep=4, scale=2.0, shared=None)),
+        pinedra_chunked_attention(heads=6, kv_heads=2, dim=32, vdim=16, scale=0.18, rot_dims=32,
+                                  base=1e6, softcap=12.0, chunk=33,
+                                  mlp=pinedra_moe(ff=24, experts=4, identity=0, top=2, groups=2,
+                                                  keep=1, scale=2.5, shared=24)),
+        pinedra_distance_attention(heads=4, kv_heads=4, dim=8, vdim=12, scale=0.35, coef=0.3,
+                                   every=500, mlp=None),
+    ])
+PINE = {"A": (PINE_A, 51, 4), "B": (PINE_B, 52, 16), "C": (PINE_C, 53, 8)}   # cfg, seed, page
+
+
+def write_pinedra_model(folder, cfg, seed, dtype, std=0.2, sharpen=3.0, router=4.0):
+    """Random weights, then the attention's query and key weights scaled up (`sharpen`), so
+    that its softmax weighs few keys heavily and a key that is lost or seen too early shows,
+    and the router's (`router`), so that the experts' scores lie apart and no choice is
+    decided by rounding."""
+    from safetensors.torch import load_file, save_file
+    from tokensprint_amd.weights import write_random_model
+    d = write_random_model(folder, cfg, seed, dtype, std=std)
+    file = next(d.glob("*.safetensors"))
+    tensors = load_file(str(file))
+    for name in tensors:
+        factor = sharpen if name.endswith((".mix.q", ".mix.k")) else \
+            router if name.endswith(".mlp.router") else 1.0
+        if factor != 1.0:
+            tensors[name] = (tensors[name].float() * factor).to(tensors[name].dtype)
+    save_file(tensors, str(file))
+    return d

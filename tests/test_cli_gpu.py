@@ -182,3 +182,23 @@ def test_run_py_serves_a_zolorax_model(gpu_device, tmp_path):
     for _ in range(9):
         tokens.append(int(zolorax_plain.forward(pcfg, w, tokens)[-1].argmax()))
     assert got == tokens[len(prompt):]
+
+
+def test_run_py_serves_a_pinedra_model(gpu_device, tmp_path):
+    """The same for Pinedra: a loop whose later passes take the embedding's output in again,
+    chunks, a distance bias, keys that serve as values, identity experts."""
+    from helpers import PINE_A
+    from plain import pinedra_plain
+    prompt = random_prompt(21, PINE_A["vocab"], 9)
+    model_dir = tmp_path / "pine-a"
+    proc = run_program(["run.py", "--config-json", config_json(tmp_path, PINE_A),
+                        "--random-weights", "2", "--model-dir", model_dir, "--dtype", "float32",
+                        "--temperature", "0", "--max-tokens", "9", "--ignore-eos", "True",
+                        "--max-num-seqs", "8", "--max-model-len", "256",
+                        "--prompt-ids", ",".join(map(str, prompt))])
+    got = json.loads(proc.stdout.strip().splitlines()[-1])
+    pcfg, w = pinedra_plain.read_model_dir(model_dir)
+    tokens = list(prompt)
+    for _ in range(9):
+        tokens.append(int(pinedra_plain.forward(pcfg, w, tokens)[-1].argmax()))
+    assert got == tokens[len(prompt):]

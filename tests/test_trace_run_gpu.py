@@ -14,9 +14,10 @@ import pytest
 import torch
 
 from drives import row_tolerance
-from helpers import PALE, TINY, ZOLO, ZONO, random_prompt, write_palelix_model, write_zolorax_model
+from helpers import (PALE, PINE, TINY, ZOLO, ZONO, random_prompt, write_palelix_model,
+                     write_pinedra_model, write_zolorax_model)
 from plain import qwen3_plain as plain
-from plain import palelix_plain, zolorax_plain, zonopel_plain
+from plain import palelix_plain, pinedra_plain, zolorax_plain, zonopel_plain
 from tokensprint_amd.weights import write_random_model
 
 pytestmark = pytest.mark.gpu
@@ -73,7 +74,7 @@ def check(got, ref, rtol, atol, what):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["B", "C", "zonopel-A", "zonopel-B", "palelix-A", "palelix-B",
-                                  "zolorax-A", "zolorax-B"])
+                                  "zolorax-A", "zolorax-B", "pinedra-A", "pinedra-B"])
 def test_replay_variants(tmp_path, name, dtype):
     stored = torch.float32 if dtype == "float32" else torch.bfloat16
     rtol, atol = TOL[dtype]
@@ -103,6 +104,16 @@ def test_replay_variants(tmp_path, name, dtype):
         pcfg, w = zolorax_plain.read_model_dir(model_dir)
         vocab = cfg["vocab"]
         forward = lambda t: zolorax_plain.forward(pcfg, w, t).float()
+        rtol, atol = max(rtol, 2e-4), max(atol, 5e-5)
+    elif name.startswith("pinedra-"):
+        if dtype == "bfloat16":
+            pytest.skip("this design's bfloat16 runs are judged by the share of rows within the "
+                        "tolerance (a router's near ties), in test_pinedra_gpu.py")
+        cfg, seed, _ = PINE[name[-1]]
+        model_dir = write_pinedra_model(tmp_path / "model", cfg, seed, stored)
+        pcfg, w = pinedra_plain.read_model_dir(model_dir)
+        vocab = cfg["vocab"]
+        forward = lambda t: pinedra_plain.forward(pcfg, w, t).float()
         rtol, atol = max(rtol, 2e-4), max(atol, 5e-5)
     else:
         cfg, seed, _ = TINY[name]
