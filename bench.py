@@ -410,6 +410,41 @@ def zolorax_configs(s):
     return config(ff), zono
 
 
+def pinedra_configs(s):
+    """(Pinedra, Zolorax) at the width, depth, vocabulary and number of matrix parameters of
+    the size `s`.  Pinedra: chunked attention with capped scores (chunks of the size's
+    window), attention whose keys are its values, attention with a distance bias, and the
+    second kind again, in turn; in every layer routed experts (7 and an identity expert, of
+    which a token uses 2, in 4 groups of which 2 are kept) beside a shared expert of twice an
+    expert's inner size, which takes up what is left."""
+    import math
+    from tokensprint_amd.weights.random_init import declared_tensors
+    hd, heads, kv = s["head_dim"], s["heads"], s["kv_heads"]
+
+    def layers(expert_ff):
+        base = {"heads": heads, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5}
+        chunked = {"type": "attention_3", "mixer": dict(
+            base, softcap=30.0, mask={"size": s["window"]}, rot={"base": 1e6, "dims": hd // 2})}
+        keys = {"type": "attention", "mixer": dict(base)}
+        distance = {"type": "attention_2", "mixer": dict(base, q_temp={"coef": 0.1, "every": 512})}
+        kinds = [chunked, keys, distance, keys]
+        mlp = {"kind": "moe", "expert": {"ff": expert_ff}, "shared": {"ff": 2 * expert_ff},
+               "router": {"experts": 7, "identity": 1, "top": 2, "scale": 2.5,
+                          "groups": {"count": 4, "keep": 2}}}
+        return [dict(kinds[i % 4], mlp=mlp) for i in range(s["layers"])]
+
+    def config(expert_ff):
+        return {"architecture": "Pinedra", "width": s["width"], "vocab": s["vocab"],
+                "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0}, "layers": layers(expert_ff)}
+
+    def count(raw):
+        return sum(math.prod(d.shape) for d in declared_tensors(raw).values())
+    zolo = zolorax_configs(s)[0]
+    spare = count(zolo) - count(config(64))
+    ff = 64 + max(0, round(spare / (3 * s["width"] * 9 * s["layers"]) / 64)) * 64
+    return config(ff), zolo
+
+
 class TimedOps:
     """Wraps a kernel provider: every call of one of its operations is bracketed by events,
     and `seconds` sums them per operation name (an eager step's kernels, one by one)."""
@@ -478,8 +513,10 @@ def zonopel_profile_step(args) -> int:
     from tokensprint_amd.engine.runner import ModelRunner
     size = COMPARE_SIZES[args.compare_size or "1b-layers"]
     zono = palelix_configs(size)[0] if args.profile_palelix else \
-        zolorax_configs(size)[0] if args.profile_zolorax else compare_configs(size)[0]
-    args.profile_zonopel = args.profile_zonopel or args.profile_palelix or args.profile_zolorax
+        zolorax_configs(size)[0] if args.profile_zolorax else \
+        pinedra_configs(size)[0] if args.profile_pinedra else compare_configs(size)[0]
+    args.profile_zonopel = args.profile_zonopel or args.profile_palelix or args.profile_zolorax \
+        or args.profile_pinedra
     _, model = random_model(zono, 0, args.dtype, "cuda:0")
     make = prefill_entries(2048) if args.profile_zonopel == "prefill" else decode_entries(8, 2048)
     lengths = make(None)
@@ -502,7 +539,8 @@ def zonopel_compare(args) -> int:
     from tokensprint_amd.engine.assemble import random_model
     page, T, b, ctx = 16, 2048, 8, 2048
     pair = ("palelix", "zonopel") if args.compare_palelix else \
-        ("zolorax", "zonopel") if args.compare_zolorax else ("zonopel", "qwen3")
+        ("zolorax", "zonopel") if args.compare_zolorax else \
+        ("pinedra", "zolorax") if args.compare_pinedra else ("zonopel", "qwen3")
     out = {"metric": f"{pair[0]} beside {pair[1]} at equal sizes (random weights, bf16)",
            "sizes": {}}
     for name, size in COMPARE_SIZES.items():
@@ -510,7 +548,8 @@ def zonopel_compare(args) -> int:
             continue
         row = {}
         configs = palelix_configs(size) if args.compare_palelix else \
-            zolorax_configs(size) if args.compare_zolorax else compare_configs(size)
+            zolorax_configs(size) if args.compare_zolorax else \
+            pinedra_configs(size) if args.compare_pinedra else compare_configs(size)
         for design, raw in zip(pair, configs):
             _, model = random_model(raw, 0, args.dtype, "cuda:0")
             vocab = size["vocab"]
@@ -569,6 +608,11 @@ def main() -> int:
     ap.add_argument("--compare-zolorax", action="store_true",
                     help="instead of the benchmark: Zolorax beside Zonopel at equal sizes "
                          "(prefill and decode throughput, time per kind of kernel)")
+    ap.add_argument("--compare-pinedra", action="store_true",
+                    help="instead of the benchmark: prefill and decode throughput of Pinedra "
+                         "beside Zolorax at equal sizes, with the time of every kind of kernel")
+    ap.add_argument("--profile-pinedra", default=None, choices=["prefill", "decode"],
+                    help="as --profile-zonopel, for the Pinedra model of --compare-size")
     ap.add_argument("--profile-zolorax", default=None, choices=["prefill", "decode"],
                     help="as --profile-zonopel, for the Zolorax model of --compare-size")
     ap.add_argument("--profile-palelix", default=None, choices=["prefill", "decode"],
@@ -585,9 +629,9 @@ def main() -> int:
     import torch
     from tokensprint_amd.config import load_named_config
 
-    if args.profile_zonopel or args.profile_palelix or args.profile_zolorax:
+    if args.profile_zonopel or args.profile_palelix or args.profile_zolorax or args.profile_pinedra:
         return zonopel_profile_step(args)
-    if args.compare_zonopel or args.compare_palelix or args.compare_zolorax:
+    if args.compare_zonopel or args.compare_palelix or args.compare_zolorax or args.compare_pinedra:
         return zonopel_compare(args)
     raw = load_named_config(args.model)
     full_layers = raw["num_hidden_layers"]

@@ -220,11 +220,11 @@ class ToyOffsetEncoding(PositionEncoding):
 
 
 class ToyScaledEmbedding(Embedding):
-    """Rows of the table times a constant (as architectures that scale their embeddings by
-    the root of the width do)."""
+    """Rows of the table times a constant, by a multiplication of the toy's own (the built-in
+    embedding has a `scale` of its own; this one's parameter is `factor`)."""
 
     def forward(self, token_ids):
-        return super().forward(token_ids) * self.params["scale"]
+        return super().forward(token_ids) * self.params["factor"]
 
 
 class ToyCappedHead(Head):
@@ -270,7 +270,7 @@ def toy_spec(raw):
     )
     return ModelSpec(
         architecture="ToyForTests", width=W, vocab_size=V,
-        embedding=PartSpec("toy_scaled_embedding", {"weight": "embed", "vocab_size": V, "scale": 3.0}),
+        embedding=PartSpec("toy_scaled_embedding", {"weight": "embed", "vocab_size": V, "factor": 3.0}),
         positions={"offset": PartSpec("toy_offset", {"step": 0.01}),
                    "rope": PartSpec("rope", {"dim": 16, "theta": 100.0, "max_position": 128})},
         layers=layers,

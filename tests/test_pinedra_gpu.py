@@ -215,6 +215,7 @@ MIXER_CASES = [
     ("attention_2", dict(heads=3, kv_heads=1, dim=16, vdim=8, scale=0.25, q_temp={"coef": 0.5, "every": 4})),
     ("attention_2", dict(heads=4, kv_heads=4, dim=48, vdim=48, scale=0.15, q_temp={"coef": 0.3, "every": 128})),
     ("attention_2", dict(heads=8, kv_heads=2, dim=24, vdim=80, scale=0.2, q_temp={"coef": 1.0, "every": 1})),
+    ("attention_2", dict(heads=2, kv_heads=1, dim=64, vdim=32, scale=0.12, q_temp={"coef": 0.2, "every": 50})),
     ("attention_3", dict(heads=4, kv_heads=2, dim=12, vdim=20, scale=0.4, softcap=5.0,
                          mask={"size": 7}, rot={"dims": 8, "base": 10000.0})),
     ("attention_3", dict(heads=4, kv_heads=1, dim=64, vdim=64, scale=0.125, softcap=20.0,
@@ -225,7 +226,8 @@ MIXER_CASES = [
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("kind, m", MIXER_CASES, ids=[f"{k}-{m['dim']}" for k, m in MIXER_CASES])
+@pytest.mark.parametrize("kind, m", MIXER_CASES,
+                         ids=[f"{k}-{m['dim']}-{m['vdim']}" for k, m in MIXER_CASES])
 def test_mixers_alone_whole_and_cut_around_chunks_and_pages(gpu_device, dtype, kind, m):
     """330 tokens over pages of 16: whole, and cut at and around page and chunk borders down to
     single tokens."""
@@ -320,8 +322,11 @@ def test_a_key_far_back_under_a_distance_bias_and_a_further_term_that_wins(gpu_d
     want = plain.attention_distance(h2.double(), w2, "x.", m_sharp, 1e-5).float()
     scene = Scene(gpu_device, part.cache_need(), 16, 1, dtype=dtype, num_pages=30)
     got = run_part_in_steps(part, h2.to(gpu_device), scene, [30] + [1] * 10)
-    torch.testing.assert_close(got, want, **(dict(rtol=5e-3, atol=5e-4) if dtype == torch.float32
-                                             else dict(rtol=6e-2, atol=3e-2)))
+    torch.testing.assert_close(got, want, **(
+        dict(rtol=5e-3, atol=5e-4) if dtype == torch.float32
+        else dict(rtol=6e-2, atol=0.05 * float(want.abs().max()))))
+    # the further term holds most of the weight: outputs are far smaller than the values
+    assert float(want.abs().mean()) < 0.5 * float((h2.double() @ w2["x.v"].T).abs().mean())
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

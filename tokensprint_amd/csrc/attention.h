@@ -41,6 +41,7 @@ __host__ __device__ __forceinline__ bool has_score_extras(const AttentionArgs& a
 
 // What turns a query row's products into scores, when there are such extras.
 struct ScoreExtra {
+  int pos;                // the query's position (distances are counted from it)
   float row_scale;        // scale times the query's temperature
   float cap, inv_cap;     // cap 0: none
   float slope;            // of the row's head; 0: none
@@ -48,6 +49,7 @@ struct ScoreExtra {
 
 __device__ __forceinline__ ScoreExtra score_extra(const AttentionArgs& a, int head, int pos) {
   ScoreExtra x;
+  x.pos = pos;
   float temp = 1.f;
   if (a.temp_every > 0)
     temp = 1.f + a.temp_coef * logf((float)((max(pos, 0) + 1) / a.temp_every + 1));
@@ -58,11 +60,20 @@ __device__ __forceinline__ ScoreExtra score_extra(const AttentionArgs& a, int he
   return x;
 }
 
-// A score from the product q . k for the key `distance` positions back.
-__device__ __forceinline__ float extra_score(const ScoreExtra& x, float dot, int distance) {
+// A score from the product q . k for the key at position `key`.  FAST: the hyperbolic
+// tangent as 1 - 2 / (exp(2 z) + 1) by the hardware's exponential and reciprocal (for
+// kernels whose operands are bfloat16; the float32 kernel takes the library's).
+template <bool FAST = false>
+__device__ __forceinline__ float extra_score(const ScoreExtra& x, float dot, int key) {
   float s = dot * x.row_scale;
-  if (x.cap > 0.f) s = x.cap * tanhf(s * x.inv_cap);
-  return s - x.slope * (float)distance;
+  if (x.cap > 0.f) {
+    const float z = s * x.inv_cap;
+    const float th = FAST ? 1.f - 2.f * __builtin_amdgcn_rcpf(
+                                      __builtin_amdgcn_exp2f(fminf(z * 2.88539008177792681f, 126.f)) + 1.f)
+                          : tanhf(z);
+    s = x.cap * th;
+  }
+  return s - x.slope * (float)(x.pos - key);
 }
 
 // The sum of a row's softmax weights with the head's sink in it.  `m_log2` is the row's

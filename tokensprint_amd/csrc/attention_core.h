@@ -252,7 +252,7 @@ __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>&
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = PERM ? kb + g * 8 + blk * 4 + i : kb + blk * 16 + g * 4 + i;
-        st[blk][i] = extra_score(*x, st[blk][i], t.pos - key) * 1.44269504088896341f;
+        st[blk][i] = extra_score<true>(*x, st[blk][i], key) * 1.44269504088896341f;
       }
     scale_log2 = 1.f;
   }

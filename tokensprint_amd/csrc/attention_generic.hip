@@ -73,7 +73,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
         } else {
           for (int d = 0; d < hd; ++d) dot = fmaf(q_s[wave][d], to_f32(kr[d]), dot);
         }
-        s = extras ? extra_score(x, dot, pos - j) : dot * a.scale;
+        s = extras ? extra_score(x, dot, j) : dot * a.scale;
       }
     }
     const float m_new = fmaxf(m, wave_max(s));

@@ -91,221 +91,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionMfmaArg
   }
 }
 
-// ---------------------------------------------------------------------------------
-// The same walk with the workgroup's four waves sharing every K and V block through LDS
-// (page sizes that are powers of two from 16 up).  The waves take four consecutive query tiles of
-// one entry and one key/value head; per block of 32 keys each wave fetches a quarter of
-// the operand registers from global memory and stores them to LDS in operand layout,
-// double-buffered: the fetch of the next block is in flight while a block is worked on,
-// and one barrier per block separates the two.  A block is read from L2 once per workgroup
-// instead of once per wave, and operands come out of LDS just before their product, so
-// few registers are held and several workgroups share a CU.
-template <int HD>
-__global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_kernel(
-    AttentionMfmaArgs args) {
-  constexpr int KS = (HD + 31) / 32, DB = HD / 16;
-  constexpr int KQ = (2 * KS + 3) / 4, VQ = (2 * DB + 3) / 4;    // operand slots per wave
-  __shared__ bf16x8 k_lds[2][2 * KS][kWave];
-  __shared__ bf16x8 v_lds[2][DB][kWave];     // low half: first 16-key block, high: second
-  const AttentionArgs& a = args.base;
-  const int wave = uniform(threadIdx.x / kWave), lane = threadIdx.x % kWave;
-  const int r = lane % 16, g = lane / 16;
-  const int group = a.nq / a.nkv;
-  const int heads = a.nkv * args.head_blocks;
-  const int head_slot = blockIdx.x % heads;                   // one head per XCD's L2
-  // All workgroups of a prompt of a few thousand tokens are resident at once, two or
-  // three to a compute unit, in launch order: the first half of the launch takes the
-  // items with the longest key ranges, longest first, the second half the shortest,
-  // shortest first, so a unit's workgroups add up to about the same work.
-  const int rank = blockIdx.x / heads, half = (args.num_tiles + 1) / 2;
-  const int item = rank < half ? rank : args.num_tiles - 1 - (rank - half);   // sorted: longest first
-  const int kvh = head_slot / args.head_blocks;
-  const int hb = head_slot % args.head_blocks;
-  const int entry = uniform(args.tiles[item * 3]), tok0 = uniform(args.tiles[item * 3 + 1]),
-            ntok = uniform(args.tiles[item * 3 + 2]);
-  const int* table = a.table + (int64_t)entry * a.table_width;
-  const int P = a.page_size;
-  const int tq = 16 / args.rows_per_token;
+#include "attention_prefill_lds_kernel.h"
 
-  // this wave's tile: tokens [wave*tq, wave*tq + tq) of the item
-  const int ti = wave * tq + r / args.rows_per_token;
-  const int hh = hb * 16 + r % args.rows_per_token;
-  const int head = kvh * group + min(hh, group - 1);
-  // (16 rows need not be a whole number of tokens: a row past the tile's tokens would be
-  // the next wave's token with this wave's key range, stored over the right result)
-  const bool row_ok = r / args.rows_per_token < tq && ti < ntok && hh < group;
-  const int pos_first = uniform(a.positions[tok0]);
-  const int pos_last = pos_first + ntok - 1;
-  const int lo_all = first_visible(a, pos_first);
-  const float scale_log2 = a.scale * 1.44269504088896341f;
-
-  TileState<HD> t;
-  t.pos = row_ok ? pos_first + ti : -1;
-  t.lo = first_visible(a, t.pos);
-  const int tile_first = pos_first + wave * tq;
-  const int tile_last = wave * tq < ntok ? pos_first + min(ntok, (wave + 1) * tq) - 1 : -1;
-  const int tile_lo = first_visible(a, tile_first);
-  const int tile_lo_last = first_visible(a, tile_last);
-  load_query<HD>(t, (const bf16_t*)a.q + ((int64_t)(tok0 + min(ti, ntok - 1)) * a.nq + head) * HD,
-                 row_ok, g);
-
-  const bf16_t* kp = (const bf16_t*)a.k_pages;
-  const bf16_t* vp = (const bf16_t*)a.v_pages;
-  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  const bf16x4 zero4 = {0, 0, 0, 0};
-  PageCursor cur{(ConstTable)table, P, pos_last, -1, -1};
-  const int key_begin = lo_all & ~31;
-  cur.start(key_begin);
-
-  // This wave's quarter of a block's operands: global -> registers.  The loads are
-  // issued unconditionally (a missing page reads page 0 and is zeroed when stored to
-  // LDS), so nothing but the barrier stands between them and the work on the block.
-  constexpr bool kEven = (2 * KS) % 4 == 0, vEven = (2 * DB) % 4 == 0;
-  // Values, wide form (head sizes in steps of 64): a block's values are DB * 16 head
-  // elements times 32 keys, 64 bytes a row of the transposed page: a lane fetches 8 keys
-  // of one row in a 16-byte load (lane % 4 = which 8 keys, lane / 4 and the instruction =
-  // which row) instead of 4 keys in an 8-byte one, half the load instructions, and the two
-  // groups of 4 keys go to their lanes' slots in LDS, every lane of a store to a bank of
-  // its own.
-  constexpr bool kWideV = DB % 4 == 0;
-  // kAhead blocks are on their way from memory while one is worked on.  More than one
-  // was measured and does not pay: the registers they take cost a resident wave, and it
-  // is the number of resident waves (four per SIMD up to head size 128) that hides the
-  // waits of this kernel, those for memory among them.
-  constexpr int kAhead = 1;
-  struct Fetched {
-    bf16x8 k[KQ];
-    bf16x4 v[VQ];
-    bf16x8 vw[kWideV ? DB / 4 : 1];             // wide form: 8 keys of one head element each
-    bool kvalid[KQ], vvalid[VQ];                // wave-uniform but for the head size's tail
-    bool vwvalid;                               // wide form: this lane's half of the block
-  };
-  Fetched ring[kAhead];
-  // address = head base + page * page stride (scalar) + position in page (scalar)
-  //           + this lane's offset inside the slot (fixed for the whole walk)
-  const int64_t k_page_stride = (int64_t)a.nkv * P * HD, v_page_stride = k_page_stride;
-  const bf16_t* k_head = kp + (int64_t)kvh * P * HD;
-  const bf16_t* v_head = vp + (int64_t)kvh * HD * P;
-  // in bytes and unsigned: added to a scalar base as a 32-bit offset, without 64-bit
-  // lane arithmetic (a page of one head is far below 4 GiB)
-  unsigned k_lane[KQ], v_lane[VQ];
-  int k_blk[KQ], v_blk[VQ];
-  bool k_dim_ok[KQ];
-#pragma unroll
-  for (int i = 0; i < KQ; ++i) {
-    const int q = kEven ? wave + 4 * i : min(wave + 4 * i, 2 * KS - 1);
-    const int s0 = q % KS;
-    k_blk[i] = q / KS;
-    k_dim_ok[i] = KS * 32 == HD || g * 8 * KS + s0 * 8 < HD;
-    k_lane[i] = 2u * (r * HD + min(g * 8 * KS + s0 * 8, HD - 8));
-  }
-  const int vw_q = lane % 4;                          // keys vw_q * 8 .. + 7 of the block
-  unsigned vw_lane[kWideV ? DB / 4 : 1];
-  if constexpr (kWideV) {
-#pragma unroll
-    for (int i = 0; i < DB / 4; ++i)
-      vw_lane[i] = 2u * ((((i * 4 + wave) * 16 + lane / 4) * P) + (vw_q % 2) * 8);
-  }
-#pragma unroll
-  for (int i = 0; i < VQ; ++i) {
-    const int q = vEven ? wave + 4 * i : min(wave + 4 * i, 2 * DB - 1);
-    v_blk[i] = q / DB;
-    v_lane[i] = 2u * (((q % DB) * 16 + r) * P + g * 4);
-  }
-  // the offset as the load sees it: opaque, so that it stays a 32-bit register beside the
-  // scalar base instead of being widened once, outside the loop, into a register pair
-  auto lane_offset = [](unsigned off) {
-    asm volatile("" : "+v"(off));
-    return off;
-  };
-  auto fetch = [&](Fetched& f, int kb) {
-    const int in_page = kb & (P - 1);             // a block of 16 keys never straddles a page
-    const int page0 = cur.next0, page1 = cur.next1;
-    const bf16_t* kb0 = k_head + (int64_t)max(page0, 0) * k_page_stride + in_page * HD;
-    const bf16_t* kb1 = k_head + (int64_t)max(page1, 0) * k_page_stride +
-                        ((in_page + 16) & (P - 1)) * HD;
-    const bf16_t* vb0 = v_head + (int64_t)max(page0, 0) * v_page_stride + in_page;
-    const bf16_t* vb1 = v_head + (int64_t)max(page1, 0) * v_page_stride + ((in_page + 16) & (P - 1));
-#pragma unroll
-    for (int i = 0; i < KQ; ++i) {
-      f.kvalid[i] = (k_blk[i] ? page1 : page0) >= 0 && k_dim_ok[i];
-      f.k[i] = *(const bf16x8*)((const char*)(k_blk[i] ? kb1 : kb0) + lane_offset(k_lane[i]));
-    }
-    if constexpr (kWideV) {
-      const bool second = vw_q >= 2;             // the block's second 16 keys
-      f.vwvalid = (second ? page1 : page0) >= 0;
-      const char* vb = (const char*)(second ? vb1 : vb0);
-#pragma unroll
-      for (int i = 0; i < DB / 4; ++i) f.vw[i] = *(const bf16x8*)(vb + vw_lane[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < VQ; ++i) {
-        f.vvalid[i] = (v_blk[i] ? page1 : page0) >= 0;
-        f.v[i] = *(const bf16x4*)((const char*)(v_blk[i] ? vb1 : vb0) + lane_offset(v_lane[i]));
-      }
-    }
-    cur.start(kb + 32);
-  };
-  // registers -> LDS, operand layout.  (Blanking under a branch, taken only by the last
-  // block of a context, was measured: slower than the selects it saves.)
-  auto stash = [&](const Fetched& f, int buf) {
-#pragma unroll
-    for (int i = 0; i < KQ; ++i)
-      if (kEven || wave + 4 * i < 2 * KS)
-        k_lds[buf][wave + 4 * i][lane] = f.kvalid[i] ? f.k[i] : zero8;
-    if constexpr (kWideV) {
-      // keys vw_q*8 .. +3 belong to lane group (vw_q % 2) * 2, the next four to the group
-      // after it, in the half of the slot that the 16-key half of the block has
-#pragma unroll
-      for (int i = 0; i < DB / 4; ++i) {
-        const bf16x8 x = f.vwvalid ? f.vw[i] : zero8;
-        const bf16x4 lo = {x[0], x[1], x[2], x[3]}, hi = {x[4], x[5], x[6], x[7]};
-        bf16x4* slot = (bf16x4*)&v_lds[buf][i * 4 + wave][(vw_q % 2) * 32 + lane / 4];
-        slot[vw_q / 2] = lo;
-        slot[32 + vw_q / 2] = hi;                 // 16 lanes further: the next lane group
-      }
-      return;
-    }
-#pragma unroll
-    for (int i = 0; i < VQ; ++i)
-      if (vEven || wave + 4 * i < 2 * DB)
-        ((bf16x4*)&v_lds[buf][(wave + 4 * i) % DB][lane])[(wave + 4 * i) / DB] =
-            f.vvalid[i] ? f.v[i] : zero4;
-  };
-
-#pragma unroll
-  for (int p = 0; p < kAhead; ++p)
-    if (key_begin + 32 * p <= pos_last) fetch(ring[p], key_begin + 32 * p);
-  stash(ring[0], 0);
-  __syncthreads();
-  int buf = 0;
-  // ring slot p holds block kb0 + 32 p, already in LDS when its turn comes, and is
-  // fetched into again at once for the block kAhead further on
-  for (int kb0 = key_begin; kb0 <= pos_last; kb0 += 32 * kAhead) {
-#pragma unroll
-    for (int p = 0; p < kAhead; ++p) {
-      const int kb = kb0 + 32 * p;
-      if (kb > pos_last) break;
-      if (kb + 32 * kAhead <= pos_last) fetch(ring[p], kb + 32 * kAhead);
-      if (kb <= tile_last && kb + 31 >= tile_lo) {
-        KvBlock<HD> b;
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-          for (int s0 = 0; s0 < KS; ++s0) b.k[blk][s0] = k_lds[buf][blk * KS + s0][lane];
-#pragma unroll
-        for (int db = 0; db < DB; ++db) b.v[db] = v_lds[buf][db][lane];
-        tile_update<HD, true>(t, b, kb, scale_log2, kb + 31 <= tile_first && kb >= tile_lo_last, g);
-      }
-      if (kb + 32 <= pos_last) stash(ring[(p + 1) % kAhead], buf ^ 1);
-      __syncthreads();
-      buf ^= 1;
-    }
-  }
-  const float sum = sum_with_sink(row_sum<HD>(t), t.m, a.sink, head);                // by all lanes: it crosses lanes
-  if (row_ok)
-    store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
-}
 
 
 // ---------------------------------------------------------------------------------
@@ -957,6 +744,7 @@ extern "C" void ts_attention_prefill_variant(int v) { g_prefill_variant = v; }
 // two items a compute unit (then eight waves share every block they bring in, and twice
 // the waves fit beside the same rings); the register-only kernel's own count otherwise.
 extern "C" int ts_attention_prefill_tiles(int head_dim, int page_size, int tiles16, int heads) {
+  if (heads < 0) return 4;      // (asked for the kernel with score extras: always four)
   if (!(page_size >= 16 && (page_size & (page_size - 1)) == 0)) return tiles_per_wave(head_dim);
   const bool wide = g_prefill_variant >= 2 && head_dim % 64 == 0 && head_dim <= 128;
   const int64_t items4 = (int64_t)((tiles16 + 3) / 4) * heads;
@@ -1056,6 +844,7 @@ static int launch_prefill(const AttentionMfmaArgs& args, hipStream_t stream) {
 }
 
 int ts_check_attention_mfma_args(const AttentionMfmaArgs& args, const char* who);
+int launch_attention_prefill_scores(const AttentionMfmaArgs& args, hipStream_t stream);
 
 // `tiles` lists wave items (entry, first flat token, tokens) of at most
 // tiles_per_wave * (16 / rows_per_token) consecutive tokens each.
@@ -1066,6 +855,14 @@ extern "C" int ts_attention_prefill(const AttentionMfmaArgs* p, hipStream_t stre
   if (ts_check_attention_mfma_args(args, "attention_prefill")) return -1;
   if (!args.tiles) TS_FAIL("attention_prefill: no tile list");
   const bool page16 = a.page_size >= 16 && (a.page_size & (a.page_size - 1)) == 0;
+  if (has_score_extras(a)) {
+    if (!page16 || args.tiles_per_wave != 4)
+      TS_FAIL("attention_prefill: scores with extras take pages of a power of two from 16 and "
+              "items of 4 tiles");
+    if (launch_attention_prefill_scores(args, stream)) return -1;
+    TS_CHECK_LAUNCH("attention_prefill");
+    return 0;
+  }
   int rc = 0;
   switch (a.hd) {
 #define TS_CASE(HD)                                                               \

@@ -739,10 +739,10 @@ class HipOps:
         extras = softcap is not None or slopes is not None or q_temp is not None
         if (q.dtype == torch.bfloat16 and cache.k_pages.dtype == torch.bfloat16
                 and head_dim % 16 == 0 and head_dim <= 256 and cache.page_size % 4 == 0):
-            # (scores with extras are the business of one matrix-core kernel and the
-            # float32 one)
-            if not extras and self._decode_fits(batch, num_kv_heads, num_heads // num_kv_heads,
-                                                head_dim, cache.page_size, False):
+            # (scores with extras: the decode kernel and the kernel for short portions and
+            # mixed steps know them, the LDS-tiled kernels for long portions do not)
+            if self._decode_fits(batch, num_kv_heads, num_heads // num_kv_heads, head_dim,
+                                 cache.page_size, False):
                 self._attention_decode(a, batch, num_heads // num_kv_heads)
             else:
                 self._attention_mfma(a, batch, num_heads // num_kv_heads, extras)
@@ -764,9 +764,8 @@ class HipOps:
         that shape instead of a tensor (the caller hands it to `linear_into_stream` or
         `linear`, or asks it for the tensor with `merged()`)."""
         T = qkv.shape[0]
-        extras = softcap is not None or slopes is not None or q_temp is not None
         fused = (qkv.dtype == torch.bfloat16 and cache.k_pages.dtype == torch.bfloat16
-                 and not extras and bool(write_cache) == bool(kv_in_row)
+                 and bool(write_cache) == bool(kv_in_row)
                  and self._decode_fits(batch, num_kv_heads, num_heads // num_kv_heads,
                                        head_dim, cache.page_size, True))
         if not fused:
@@ -788,7 +787,7 @@ class HipOps:
         out = torch.empty(T, num_heads, head_dim, dtype=qkv.dtype, device=self.device)
         a = AttentionArgs()
         self._fill_attention_args(a, None, out, batch, table, cache, num_heads, num_kv_heads,
-                                  head_dim, scale, window, sink, chunk)
+                                  head_dim, scale, window, sink, chunk, softcap, slopes, q_temp)
         if sink is not None or chunk is not None:
             defer_merge = False        # the product that merges for itself knows neither
         d = AttentionDecodeArgs()
@@ -862,10 +861,13 @@ class HipOps:
         m.base = a
         m.rows_per_token, m.head_blocks = rows_per_token, head_blocks
         # long portions of prompts: a wavefront takes several query tiles and walks alone
-        if not extras and self._prefill_tiles(batch, a.nkv, group) is not None:
+        # (scores with extras: the one of those kernels that knows them takes pages of a power
+        # of two from 16 and asks for items of four tiles, which a head count of -1 says)
+        page16 = a.page_size >= 16 and a.page_size & (a.page_size - 1) == 0
+        if (not extras or page16) and self._prefill_tiles(batch, a.nkv, group) is not None:
             tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
             tpw = self.lib.ts_attention_prefill_tiles(a.hd, a.page_size, tiles16,
-                                                      a.nkv * head_blocks)
+                                                      -1 if extras else a.nkv * head_blocks)
             tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile * tpw,
                                                          longest_first=True)
             m.tiles, m.num_tiles, m.tiles_per_wave = tiles_dev.data_ptr(), num_tiles, tpw
