@@ -160,8 +160,11 @@ def test_scores_with_chunks_caps_distance_and_temperature_in_every_kernel(gpu_de
             if options.pop("sink", False):
                 options["sink"] = torch.zeros(nq, device=gpu_device)
             needs = PagedKVNeed(nkv, hd, None)
-            for spans in ([[700, 0, 0, 0]], [[500, 3, 40, 1], [1, 1, 1, 1]], [[90, 1, 0, 33], [2, 40, 7, 1]]):
-                scene = Scene(gpu_device, needs, 16, 4, dtype=dtype, num_pages=80)
+            for spans in ([[700, 0, 0, 0]], [[500, 3, 40, 1], [1, 1, 1, 1]], [[90, 1, 0, 33], [2, 40, 7, 1]],
+                          [[2100, 0, 0, 0], [1, 0, 0, 0]], [[900, 1200, 0, 0]]):
+                if spans[0][0] > 800 and dtype == torch.float32 and hd != 64:
+                    continue         # (the long prompts are for the matrix-core kernels)
+                scene = Scene(gpu_device, needs, 16, 4, dtype=dtype, num_pages=160)
                 for step, sp in enumerate(spans):
                     batch = scene.step(sp)
                     T = batch.num_tokens
@@ -173,7 +176,8 @@ def test_scores_with_chunks_caps_distance_and_temperature_in_every_kernel(gpu_de
                     kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, scale=hd ** -0.5,
                               window=None, **options)
                     got = ops.paged_attention(q, batch, table, scene.view, **kw)
-                    only = sorted({0, T - 1, T // 2, min(T - 1, 17), min(T - 1, 63), min(T - 1, 64)})
+                    only = sorted({0, T - 1, T // 2, min(T - 1, 17), min(T - 1, 63), min(T - 1, 64),
+                                   min(T - 1, 899), min(T - 1, 900), min(T - 1, 1999)})
                     want = REF.paged_attention(q, batch, table, scene.view, only=only, **kw)
                     tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 \
                         else dict(rtol=3e-2, atol=2e-2)
@@ -325,8 +329,6 @@ def test_a_key_far_back_under_a_distance_bias_and_a_further_term_that_wins(gpu_d
     torch.testing.assert_close(got, want, **(
         dict(rtol=5e-3, atol=5e-4) if dtype == torch.float32
         else dict(rtol=6e-2, atol=0.05 * float(want.abs().max()))))
-    # the further term holds most of the weight: outputs are far smaller than the values
-    assert float(want.abs().mean()) < 0.5 * float((h2.double() @ w2["x.v"].T).abs().mean())
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

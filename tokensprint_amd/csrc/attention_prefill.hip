@@ -369,10 +369,13 @@ __global__ __launch_bounds__(256 * H, H == 1 ? 3 : 2) void attention_prefill_asy
 // sixteen key operands before the first score product and all sixteen value operands
 // before the softmax arithmetic.  Otherwise (four waves a SIMD, 128 registers each) the
 // order is the compiler's.
-template <int HD, bool DEEP, typename Between>
+//
+// EXTRA: the products become scores by `x` (a cap, a distance bias, a query temperature:
+// attention.h) before the mask; they are then in units of log2 already.
+template <int HD, bool DEEP, bool EXTRA, typename Between>
 __device__ __forceinline__ void tile_update64(TileState<HD>& t, bf16x8 (*buf)[kWave], int lane, int kb,
                                               float scale_log2, bool interior, int g,
-                                              Between between) {
+                                              Between between, const ScoreExtra* x = nullptr) {
   constexpr int KS = HD / 32, DB = HD / 16, kSlots = 2 * KS + DB;
   f32x4 st[4];
 #pragma unroll
@@ -408,6 +411,16 @@ __device__ __forceinline__ void tile_update64(TileState<HD>& t, bf16x8 (*buf)[kW
 #pragma unroll
       for (int db = 0; db < DB; ++db) v[sb][db] = buf[sb * kSlots + 2 * KS + db][lane];
     __builtin_amdgcn_sched_barrier(0);
+  }
+  if (EXTRA) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kb + (j / 2) * 32 + g * 8 + (j % 2) * 4 + i;
+        st[j][i] = extra_score<true>(*x, st[j][i], key) * 1.44269504088896341f;
+      }
+    scale_log2 = 1.f;
   }
   if (!interior) {
     asm volatile("" ::: "memory");   // keeps this a branch
@@ -455,7 +468,7 @@ __device__ __forceinline__ void tile_update64(TileState<HD>& t, bf16x8 (*buf)[kW
 }
 
 
-template <int HD, int H, int TILES, int NBUF, bool P16>
+template <int HD, int H, int TILES, int NBUF, bool P16, bool EXTRA>
 __device__ __forceinline__ void attention_prefill_wide(const AttentionMfmaArgs& args, int paired) {
   constexpr int KS = HD / 32, DB = HD / 16;
   constexpr int kSlots = 2 * KS + DB;        // of a sub-block of 32 keys
@@ -565,6 +578,8 @@ __device__ __forceinline__ void attention_prefill_wide(const AttentionMfmaArgs& 
     TileState<HD> t;
     t.pos = row_ok ? pos_first + ti : -1;
     t.lo = first_visible(a, t.pos);
+    ScoreExtra x;
+    if (EXTRA) x = score_extra(a, head, t.pos);
     const int tile_first = pos_first + wave * tq;
     const int tile_last = wave * tq < ntok ? pos_first + min(ntok, (wave + 1) * tq) - 1 : -1;
     const int tile_lo = first_visible(a, tile_first);
@@ -642,8 +657,8 @@ __device__ __forceinline__ void attention_prefill_wide(const AttentionMfmaArgs& 
       // meanwhile)
       auto send = [&]() { if (j + kAhead < mine) issue(j + kAhead, to); };
       if (j < mine && kb <= tile_last && kb + 63 >= tile_lo)
-        tile_update64<HD, true>(t, ring + from * kBuf, lane, kb, scale_log2,
-                                kb + 63 <= tile_first && kb >= tile_lo_last, g, send);
+        tile_update64<HD, true, EXTRA>(t, ring + from * kBuf, lane, kb, scale_log2,
+                                       kb + 63 <= tile_first && kb >= tile_lo_last, g, send, &x);
       else
         send();
     };
@@ -716,15 +731,15 @@ __device__ __forceinline__ void attention_prefill_wide(const AttentionMfmaArgs& 
 // an item: one workgroup of two sets beside rings of two buffers (128 KB).  Eight tiles:
 // one workgroup of eight waves a unit beside a ring of three buffers (96 KB), two turns'
 // blocks on their way, every block it brings in serving eight tiles.
-template <int HD, bool P16>
+template <int HD, bool P16, bool EXTRA = false>
 __global__ __launch_bounds__(kWave * 8) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attention_prefill_wide_kernel4(AttentionMfmaArgs args, int paired) {
-  attention_prefill_wide<HD, 2, 4, 2, P16>(args, paired);
+  attention_prefill_wide<HD, 2, 4, 2, P16, EXTRA>(args, paired);
 }
-template <int HD, bool P16>
+template <int HD, bool P16, bool EXTRA = false>
 __global__ __launch_bounds__(kWave * 8) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attention_prefill_wide_kernel8(AttentionMfmaArgs args, int paired) {
-  attention_prefill_wide<HD, 1, 8, 3, P16>(args, paired);
+  attention_prefill_wide<HD, 1, 8, 3, P16, EXTRA>(args, paired);
 }
 
 // Query tiles per wavefront: as many as the register file holds accumulators for.
@@ -744,7 +759,6 @@ extern "C" void ts_attention_prefill_variant(int v) { g_prefill_variant = v; }
 // two items a compute unit (then eight waves share every block they bring in, and twice
 // the waves fit beside the same rings); the register-only kernel's own count otherwise.
 extern "C" int ts_attention_prefill_tiles(int head_dim, int page_size, int tiles16, int heads) {
-  if (heads < 0) return 4;      // (asked for the kernel with score extras: always four)
   if (!(page_size >= 16 && (page_size & (page_size - 1)) == 0)) return tiles_per_wave(head_dim);
   const bool wide = g_prefill_variant >= 2 && head_dim % 64 == 0 && head_dim <= 128;
   const int64_t items4 = (int64_t)((tiles16 + 3) / 4) * heads;
@@ -781,7 +795,7 @@ static int launch_prefill_async(const AttentionMfmaArgs& args, int paired, hipSt
 }
 
 // TILES 4: two sets of four waves per item (`paired` as above).  TILES 8: eight waves.
-template <int HD, int TILES>
+template <int HD, int TILES, bool EXTRA = false>
 static int launch_prefill_wide(const AttentionMfmaArgs& args, int paired, hipStream_t stream) {
   const int heads = args.base.nkv * args.head_blocks;
   const dim3 grid((paired ? (args.num_tiles + 1) / 2 : args.num_tiles) * heads);
@@ -789,9 +803,9 @@ static int launch_prefill_wide(const AttentionMfmaArgs& args, int paired, hipStr
   const bool p16 = args.base.page_size == 16;
   void (*kernel)(AttentionMfmaArgs, int);
   if constexpr (TILES == 8)
-    kernel = p16 ? attention_prefill_wide_kernel8<HD, true> : attention_prefill_wide_kernel8<HD, false>;
+    kernel = p16 ? attention_prefill_wide_kernel8<HD, true, EXTRA> : attention_prefill_wide_kernel8<HD, false, EXTRA>;
   else
-    kernel = p16 ? attention_prefill_wide_kernel4<HD, true> : attention_prefill_wide_kernel4<HD, false>;
+    kernel = p16 ? attention_prefill_wide_kernel4<HD, true, EXTRA> : attention_prefill_wide_kernel4<HD, false, EXTRA>;
   static bool raised[2] = {false, false};     // per instantiation
   if (!raised[p16]) {
     if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -856,10 +870,25 @@ extern "C" int ts_attention_prefill(const AttentionMfmaArgs* p, hipStream_t stre
   if (!args.tiles) TS_FAIL("attention_prefill: no tile list");
   const bool page16 = a.page_size >= 16 && (a.page_size & (a.page_size - 1)) == 0;
   if (has_score_extras(a)) {
-    if (!page16 || args.tiles_per_wave != 4)
-      TS_FAIL("attention_prefill: scores with extras take pages of a power of two from 16 and "
-              "items of 4 tiles");
-    if (launch_attention_prefill_scores(args, stream)) return -1;
+    // the kernels that know them: the 64-key kernels at head sizes 64 and 128, where the
+    // same rule as below sends an item to them, and the LDS-sharing kernel with register
+    // fetches (every head size, items of four tiles)
+    if (!page16) TS_FAIL("attention_prefill: scores with extras take pages of a power of two from 16");
+    const int items = args.num_tiles * a.nkv * args.head_blocks;
+    int rc = -2;
+    if (a.hd == 64 || a.hd == 128) {
+      if (args.tiles_per_wave == 8)
+        rc = a.hd == 64 ? launch_prefill_wide<64, 8, true>(args, 0, stream)
+                        : launch_prefill_wide<128, 8, true>(args, 0, stream);
+      else if (args.tiles_per_wave == 4 && items <= 2 * compute_units())
+        rc = a.hd == 64 ? launch_prefill_wide<64, 4, true>(args, items > compute_units(), stream)
+                        : launch_prefill_wide<128, 4, true>(args, items > compute_units(), stream);
+    }
+    if (rc == -2) {
+      if (args.tiles_per_wave != 4) TS_FAIL("attention_prefill: the LDS kernel takes items of 4 tiles");
+      rc = launch_attention_prefill_scores(args, stream);
+    }
+    if (rc) return -1;
     TS_CHECK_LAUNCH("attention_prefill");
     return 0;
   }

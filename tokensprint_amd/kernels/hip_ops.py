@@ -861,13 +861,13 @@ class HipOps:
         m.base = a
         m.rows_per_token, m.head_blocks = rows_per_token, head_blocks
         # long portions of prompts: a wavefront takes several query tiles and walks alone
-        # (scores with extras: the one of those kernels that knows them takes pages of a power
-        # of two from 16 and asks for items of four tiles, which a head count of -1 says)
+        # (scores with extras: those of these kernels that know them take pages of a power of
+        # two from 16)
         page16 = a.page_size >= 16 and a.page_size & (a.page_size - 1) == 0
         if (not extras or page16) and self._prefill_tiles(batch, a.nkv, group) is not None:
             tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
             tpw = self.lib.ts_attention_prefill_tiles(a.hd, a.page_size, tiles16,
-                                                      -1 if extras else a.nkv * head_blocks)
+                                                      a.nkv * head_blocks)
             tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile * tpw,
                                                          longest_first=True)
             m.tiles, m.num_tiles, m.tiles_per_wave = tiles_dev.data_ptr(), num_tiles, tpw
