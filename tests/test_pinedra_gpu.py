@@ -42,7 +42,10 @@ def test_finish_projection(gpu_device, out_dtype):
     for T, q_cols, k_cols, v_cols, extra, from_keys, normed, biased in (
             (5, 64, 32, 32, 8, False, False, True), (70, 48, 16, 16, 48, True, True, True),
             (1, 512, 128, 128, 0, True, True, False), (33, 16, 16, 32, 16, False, True, True),
-            (9, 1280, 256, 256, 1280, True, True, True)):
+            (9, 1280, 256, 256, 1280, True, True, True),
+            # (parts that do not begin at multiples of four columns, and rows beyond what a
+            # workgroup keeps in registers: the kernel that walks a row three times)
+            (6, 18, 6, 6, 3, True, True, True), (3, 12288, 2048, 2048, 4096, False, True, True)):
         in_ld = q_cols + k_cols + (0 if from_keys else v_cols) + extra
         rows = rnd((T, in_ld), 1, 2.0).to(gpu_device)
         bias = rnd((in_ld - extra,), 2).to(gpu_device) if biased else None
