@@ -114,6 +114,7 @@ def attention_keys_as_values(h, w, pre, m, eps):
     per output coordinate; biases on q, k and o."""
     T = h.shape[0]
     H, G, d = int(m["heads"]), int(m["kv_heads"]), int(m["dim"])
+    assert int(m.get("vdim", d)) == d
     q = linear(h, w, pre, "q", True)
     k = linear(h, w, pre, "k", True)
     v = k.reshape(T, G, d)
@@ -135,9 +136,10 @@ def attention_distance(h, w, pre, m, eps):
     k = unit_rms(linear(h, w, pre, "k").reshape(T, G, d), eps) * w[pre + "k.norm"]
     v = linear(h, w, pre, "v").reshape(T, G, dv)
     pos = torch.arange(T)
-    steps = torch.div(pos + 1, int(m["q_temp"]["every"]), rounding_mode="floor")
-    temp = 1.0 + float(m["q_temp"]["coef"]) * torch.log(steps.to(h.dtype) + 1.0)
-    q = q * temp[:, None, None]
+    if m.get("q_temp") is not None:
+        steps = torch.div(pos + 1, int(m["q_temp"]["every"]), rounding_mode="floor")
+        temp = 1.0 + float(m["q_temp"]["coef"]) * torch.log(steps.to(h.dtype) + 1.0)
+        q = q * temp[:, None, None]
     slope = torch.tensor([2.0 ** (-8.0 * (j + 1) / H) for j in range(H)], dtype=h.dtype)
     distance = (pos[:, None] - pos[None, :]).to(h.dtype)
     seen = causal_mask(T)
@@ -157,15 +159,17 @@ def attention_chunked(h, w, pre, m, eps):
     T = h.shape[0]
     H, G, d, dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
     pos = torch.arange(T)
-    q = rotate_first(linear(h, w, pre, "q", True).reshape(T, H, d), m["rot"], pos)
-    k = rotate_first(linear(h, w, pre, "k", True).reshape(T, G, d), m["rot"], pos)
+    q = linear(h, w, pre, "q", True).reshape(T, H, d)
+    k = linear(h, w, pre, "k", True).reshape(T, G, d)
+    if m.get("rot") is not None:
+        q, k = rotate_first(q, m["rot"], pos), rotate_first(k, m["rot"], pos)
     v = linear(h, w, pre, "v", True).reshape(T, G, dv)
-    cap = float(m["softcap"])
-    seen = causal_mask(T, int(m["mask"]["size"]))
+    cap = float(m["softcap"]) if m.get("softcap") is not None else None
+    seen = causal_mask(T, int(m["mask"]["size"]) if m.get("mask") is not None else None)
 
     def weights_of(s):
         s = s * float(m["scale"])
-        return softmax_rows(cap * torch.tanh(s / cap), seen)
+        return softmax_rows(s if cap is None else cap * torch.tanh(s / cap), seen)
 
     o = heads_attend(q, k, v, weights_of).reshape(T, H, dv)
     o = o * sigmoid(linear(h, w, pre, "g"))[:, :, None]

@@ -136,8 +136,8 @@ def test_every_run_owns_a_cache_and_tensors_follow_the_mixer():
     (lambda c: c["layers"][0].update(type="attention_4"), "type"),
     (lambda c: c["layers"][1]["mixer"].update(vdim=16), "vdim"),
     (lambda c: c["layers"][0]["mixer"]["rot"].update(dims=14), "rot.dims"),
-    (lambda c: c["layers"][0]["mixer"].pop("softcap"), "softcap"),
-    (lambda c: c["layers"][2]["mixer"].pop("q_temp"), "q_temp"),
+    (lambda c: c["layers"][0]["mixer"].update(softcap=-1.0), "softcap"),
+    (lambda c: c["layers"][2]["mixer"]["q_temp"].update(every=0), "q_temp"),
     (lambda c: c["layers"][0]["mixer"].update(kv_heads=3), "multiple"),
     (lambda c: c["layers"][0]["mlp"]["router"]["groups"].update(count=4), "groups"),
     (lambda c: c["layers"][0]["mlp"]["router"].update(top=5), "cannot give"),
@@ -150,6 +150,26 @@ def test_config_errors(change, message):
     change(cfg)
     with pytest.raises(ConfigError, match=message):
         PinedraConfig.from_dict(cfg)
+
+
+def test_a_constant_that_is_left_out_takes_its_mechanism_along(tmp_path):
+    """No cap, no chunks, no rotation, no temperature, a value size that the keys give: the
+    engine and the plain implementation agree on what is left."""
+    cfg = copy.deepcopy(PINE_A)
+    for key in ("softcap", "mask", "rot"):
+        cfg["layers"][0]["mixer"].pop(key)
+    cfg["layers"][3]["mixer"].pop("softcap")
+    cfg["layers"][1]["mixer"].pop("vdim")
+    cfg["layers"][2]["mixer"].pop("q_temp")
+    parsed = PinedraConfig.from_dict(cfg)
+    assert parsed.layers[0].mixer.chunk is None and parsed.layers[0].mixer.rot_dims is None
+    assert parsed.layers[1].mixer.vdim == 12 and parsed.layers[2].mixer.temp_every is None
+    d = write_pinedra_model(tmp_path, cfg, 3, torch.float32)
+    pcfg, w = plain.read_model_dir(d)
+    _, model = load_model(d, "float32", "cpu", ops=TorchOps())
+    requests = {"a": random_prompt(30, cfg["vocab"], 1), "b": random_prompt(9, cfg["vocab"], 2)}
+    ref = {rid: plain.forward(pcfg, w, t).float() for rid, t in requests.items()}
+    drives.compare(drives.drive_portions(runner_for(model, 4, 20), requests), ref, *TOL)
 
 
 # ------------------------------------------------------------------ the plain implementation's pins

@@ -125,30 +125,36 @@ class PinedraConfig:
 
     @staticmethod
     def _attention(kind, m, where) -> AttentionSizes:
+        dim = _pos_int(m, "dim", where)
         base = dict(kind=kind, heads=_pos_int(m, "heads", where),
-                    kv_heads=_pos_int(m, "kv_heads", where), dim=_pos_int(m, "dim", where),
-                    vdim=_pos_int(m, "vdim", where),
+                    kv_heads=_pos_int(m, "kv_heads", where), dim=dim,
+                    vdim=_pos_int(m, "vdim", where) if "vdim" in m or kind != "attention" else dim,
                     scale=_number(m, "scale", where, positive=True))
         if base["heads"] % base["kv_heads"]:
             raise ConfigError(f"config.json: {where}: heads={base['heads']} is not a multiple "
                               f"of kv_heads={base['kv_heads']}")
+        # (a constant that config.json leaves out: the mechanism it belongs to is not there)
         if kind == "attention":
             if base["vdim"] != base["dim"]:
                 raise ConfigError(f"config.json: {where}: the keys are the values, so vdim="
                                   f"{base['vdim']} must equal dim={base['dim']}")
         elif kind == "attention_2":
-            t = _need(m, "q_temp", where)
-            base.update(temp_coef=_number(t, "coef", where + ".q_temp"),
-                        temp_every=_pos_int(t, "every", where + ".q_temp"))
+            t = m.get("q_temp")
+            if t is not None:
+                base.update(temp_coef=_number(t, "coef", where + ".q_temp"),
+                            temp_every=_pos_int(t, "every", where + ".q_temp"))
         else:
-            rot = _need(m, "rot", where)
-            base.update(rot_base=_number(rot, "base", where + ".rot", positive=True),
-                        rot_dims=_pos_int(rot, "dims", where + ".rot"),
-                        softcap=_number(m, "softcap", where, positive=True),
-                        chunk=_pos_int(_need(m, "mask", where), "size", where + ".mask"))
-            if base["rot_dims"] % 2 or base["rot_dims"] > base["dim"]:
-                raise ConfigError(f"config.json: {where}.rot.dims={base['rot_dims']} must be "
-                                  f"even and at most dim={base['dim']}")
+            rot, mask = m.get("rot"), m.get("mask")
+            if rot is not None:
+                base.update(rot_base=_number(rot, "base", where + ".rot", positive=True),
+                            rot_dims=_pos_int(rot, "dims", where + ".rot"))
+                if base["rot_dims"] % 2 or base["rot_dims"] > base["dim"]:
+                    raise ConfigError(f"config.json: {where}.rot.dims={base['rot_dims']} must be "
+                                      f"even and at most dim={base['dim']}")
+            if m.get("softcap") is not None:
+                base.update(softcap=_number(m, "softcap", where, positive=True))
+            if mask is not None:
+                base.update(chunk=_pos_int(mask, "size", where + ".mask"))
         return AttentionSizes(**base)
 
     @staticmethod

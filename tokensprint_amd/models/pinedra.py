@@ -31,16 +31,18 @@ def _mixer_spec(m: AttentionSizes, pre: str, cfg: PinedraConfig, positions: dict
         p.update(values="keys", qk_norm="projection", bias=("q", "k", "o"), gate=True)
     elif m.kind == "attention_2":
         p.update(qk_norm=True, gate=True, sink="zero", distance_bias=SLOPE_POWER,
-                 q_temp=(m.temp_coef, m.temp_every))
+                 q_temp=(m.temp_coef, m.temp_every) if m.temp_every is not None else None)
     else:
-        head = SoftmaxAttention.padded_head(m.dim, m.vdim)
-        # one table per (base, rotated dimensions, head size), shared by the layers that use it
-        name = f"rot_{m.rot_base!r}_{m.rot_dims}_{head}"
-        positions.setdefault(name, PartSpec("rope_partial", {
-            "dims": m.rot_dims, "base": m.rot_base, "head_dim": head,
-            "max_position": cfg.max_position}))
-        p.update(position=name, bias=("q", "k", "v"), gate="head", softcap=m.softcap,
-                 chunk=m.chunk)
+        if m.rot_dims is not None:
+            head = SoftmaxAttention.padded_head(m.dim, m.vdim)
+            # one table per (base, rotated dimensions, head size), shared by the layers that
+            # use it
+            name = f"rot_{m.rot_base!r}_{m.rot_dims}_{head}"
+            positions.setdefault(name, PartSpec("rope_partial", {
+                "dims": m.rot_dims, "base": m.rot_base, "head_dim": head,
+                "max_position": cfg.max_position}))
+            p.update(position=name)
+        p.update(bias=("q", "k", "v"), gate="head", softcap=m.softcap, chunk=m.chunk)
     return PartSpec("softmax_attention", p)
 
 
