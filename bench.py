@@ -429,7 +429,7 @@ def pinedra_configs(s):
         distance = {"type": "attention_2", "mixer": dict(base, q_temp={"coef": 0.1, "every": 512})}
         kinds = [chunked, keys, distance, keys]
         mlp = {"kind": "moe", "expert": {"ff": expert_ff}, "shared": {"ff": 2 * expert_ff},
-               "router": {"experts": 7, "identity": 1, "top": 2, "scale": 2.5,
+               "router": {"experts": 7, "identity": 1, "top": 2, "scale": 2.0,
                           "groups": {"count": 4, "keep": 2}}}
         return [dict(kinds[i % 4], mlp=mlp) for i in range(s["layers"])]
 

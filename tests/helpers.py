@@ -444,8 +444,8 @@ PINE_C = pinedra_config(
         pinedra_chunked_attention(heads=6, kv_heads=2, dim=32, vdim=16, scale=0.18, rot_dims=32,
                                   base=1e6, softcap=12.0, chunk=33,
                                   mlp=pinedra_moe(ff=24, experts=4, identity=0, top=2, groups=2,
-                                                  keep=1, scale=2.5, shared=24)),
-        pinedra_distance_attention(heads=4, kv_heads=4, dim=8, vdim=12, scale=0.35, coef=0.3,
+                                                  keep=1, scale=2.25, shared=24)),
+        pinedra_distance_attention(heads=4, kv_heads=4, dim=8, vdim=12, scale=0.35, coef=0.35,
                                    every=500, mlp=None),
     ])
 PINE = {"A": (PINE_A, 51, 4), "B": (PINE_B, 52, 16), "C": (PINE_C, 53, 8)}   # cfg, seed, page

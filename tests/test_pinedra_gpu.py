@@ -116,7 +116,7 @@ def test_rows_that_enter_the_stream(gpu_device):
 
 def test_router_with_a_correction_and_experts_without_weights(gpu_device):
     ops = load_hip_ops(gpu_device)
-    for T, n, top, groups, keep, scale in ((40, 14, 3, 2, 1, 2.5), (7, 6, 2, 3, 2, 1.0),
+    for T, n, top, groups, keep, scale in ((40, 15, 4, 3, 1, 1.75), (7, 6, 2, 3, 2, 1.0),
                                            (100, 64, 8, 8, 4, 0.5), (3, 4, 4, 4, 4, 2.0), (9, 5, 1, 1, 1, 1.0)):
         logits = rnd((T, n), 1, 2.0).to(gpu_device)
         corr = (rnd((n,), 2, 0.2) - 0.3).to(gpu_device)       # most choice scores are negative
@@ -133,7 +133,7 @@ def test_router_with_a_correction_and_experts_without_weights(gpu_device):
             assert bool(((got != 0) != (bare != 0)).any())
     for dtype in (torch.float32, torch.bfloat16):
         for T, experts, identity, inner, shared in ((9, 5, 1, 12, 20), (40, 8, 0, 16, 16),
-                                                    (3, 2, 2, 7, 0), (130, 12, 2, 96, 96)):
+                                                    (3, 2, 2, 7, 0), (130, 10, 2, 88, 104)):
             weights = torch.relu(rnd((T, experts + identity), 3)).to(gpu_device)
             gate_up = rnd((T, 2 * (experts * inner + shared)), 4).to(dtype).to(gpu_device)
             kw = dict(form="silu", experts=experts, shared_inner=shared)
@@ -152,9 +152,9 @@ def test_scores_with_chunks_caps_distance_and_temperature_in_every_kernel(gpu_de
     ops = load_hip_ops(gpu_device)
     for dtype in (torch.float32, torch.bfloat16):
         for nq, nkv, hd, options in (
-                (4, 2, 64, dict(chunk=64, softcap=20.0)), (8, 8, 128, dict(chunk=1)),
+                (4, 2, 64, dict(chunk=48, softcap=15.0)), (8, 8, 128, dict(chunk=1)),
                 (6, 1, 96, dict(q_temp=(0.3, 3), sink=True, slopes=True)),
-                (2, 2, 48, dict(chunk=100, softcap=1.5, slopes=True, q_temp=(1.0, 128), sink=True)),
+                (2, 2, 48, dict(chunk=100, softcap=1.5, slopes=True, q_temp=(1.0, 96), sink=True)),
                 (4, 4, 64, dict(slopes=True)), (4, 1, 128, dict(chunk=7))):
             options = dict(options)
             if options.pop("slopes", False):
@@ -217,16 +217,16 @@ def mixer_part(gpu_device, dtype, kind, width, **m):
 
 MIXER_CASES = [
     ("attention", dict(heads=4, kv_heads=2, dim=12, vdim=12, scale=0.3)),
-    ("attention", dict(heads=2, kv_heads=1, dim=64, vdim=64, scale=0.125)),
+    ("attention", dict(heads=6, kv_heads=3, dim=64, vdim=64, scale=0.1)),
     ("attention", dict(heads=3, kv_heads=3, dim=40, vdim=40, scale=0.2)),
     ("attention_2", dict(heads=3, kv_heads=1, dim=16, vdim=8, scale=0.25, q_temp={"coef": 0.5, "every": 4})),
-    ("attention_2", dict(heads=4, kv_heads=4, dim=48, vdim=48, scale=0.15, q_temp={"coef": 0.3, "every": 128})),
+    ("attention_2", dict(heads=4, kv_heads=2, dim=48, vdim=48, scale=0.15, q_temp={"coef": 0.25, "every": 96})),
     ("attention_2", dict(heads=8, kv_heads=2, dim=24, vdim=80, scale=0.2, q_temp={"coef": 1.0, "every": 1})),
     ("attention_2", dict(heads=2, kv_heads=1, dim=64, vdim=32, scale=0.12, q_temp={"coef": 0.2, "every": 50})),
     ("attention_3", dict(heads=4, kv_heads=2, dim=12, vdim=20, scale=0.4, softcap=5.0,
                          mask={"size": 7}, rot={"dims": 8, "base": 10000.0})),
-    ("attention_3", dict(heads=4, kv_heads=1, dim=64, vdim=64, scale=0.125, softcap=20.0,
-                         mask={"size": 64}, rot={"dims": 16, "base": 1e6})),
+    ("attention_3", dict(heads=8, kv_heads=2, dim=64, vdim=64, scale=0.11, softcap=15.0,
+                         mask={"size": 48}, rot={"dims": 32, "base": 5e5})),
     ("attention_3", dict(heads=9, kv_heads=3, dim=32, vdim=16, scale=0.3, softcap=2.0,
                          mask={"size": 100}, rot={"dims": 32, "base": 300.0})),
 ]
@@ -341,7 +341,7 @@ def test_routed_feed_forward_alone(gpu_device, dtype):
     h = rnd((T, width), 2).to(dtype)
     for experts, identity, top, groups, keep, scale, shared, inner in (
             (5, 1, 2, 3, 2, 1.5, 20, 12), (8, 0, 1, 1, 1, 1.0, 16, 16), (3, 3, 3, 2, 2, 0.7, 8, 20),
-            (2, 2, 4, 4, 4, 2.0, None, 8), (12, 2, 3, 2, 1, 2.5, 96, 96)):
+            (2, 2, 4, 4, 4, 2.0, None, 8), (10, 2, 3, 3, 2, 1.75, 64, 80)):
         moe = build_part(FEED_FORWARDS, PartSpec("routed_experts", {
             "prefix": "m.", "inner_dim": inner, "experts": experts, "top": top,
             "group_count": groups, "group_keep": keep, "scores": "softmax", "normalize": False,

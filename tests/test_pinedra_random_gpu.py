@@ -30,7 +30,7 @@ def draw_mlp(rnd):
     keep = rnd.randint(1, groups)
     return pinedra_moe(ff=rnd.choice([8, 12, 40, 100]), experts=outputs - identity,
                        identity=identity, top=rnd.randint(1, min(keep * per, 4)), groups=groups,
-                       keep=keep, scale=rnd.choice([1.0, 2.5, 0.3]),
+                       keep=keep, scale=rnd.choice([1.0, 1.75, 0.3]),
                        shared=rnd.choice([None, 8, 40, 96]))
 
 
@@ -47,7 +47,7 @@ def draw_layer(rnd):
     if kind == "attention_2":
         return pinedra_distance_attention(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=scale,
                                           coef=rnd.choice([0.1, 0.5, 1.0]),
-                                          every=rnd.choice([1, 3, 16, 128]), mlp=mlp)
+                                          every=rnd.choice([1, 3, 16, 96]), mlp=mlp)
     return pinedra_chunked_attention(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=scale,
                                      rot_dims=rnd.choice([2, dim // 2 * 2, dim // 4 * 2 or 2]),
                                      base=rnd.choice([100.0, 1e4, 1e6]),
